@@ -1,0 +1,156 @@
+/*
+ * mamba2_hip.h -- C ABI of the MI355X (gfx950) Mamba-2 mixer hot path.
+ *
+ * One shared library, libmamba2_hip.so, exports the entry points below.  They
+ * replace the device kernels of awslabs/state-space-models-neuron (NKI kernels
+ * behind torch.autograd.Function wrappers; the reference has no FFI of its own,
+ * so the "binding" a maintainer adds is a ctypes call from those wrappers):
+ *
+ *   m2_conv1d_fwd / m2_conv1d_bwd      <- mamba2/conv1d_grouped.py:66-125 (conv1d_with_transpose),
+ *                                         :129-194 (conv1d_with_transpose_bwd), :198-262
+ *                                         (conv1d_grouped_kernel_grad); wrappers :265-334
+ *   m2_ssd_fwd / m2_ssd_bwd            <- mamba2/mamba2_kernel.py:67-170 (mamba_kernel_),
+ *                                         :277-485 (mamba_kernel_bwd_); wrapper :488-519
+ *   m2_decode_step                     <- mamba2/mamba2_kernel_inference.py:27-104
+ *                                         (mamba_inference_kernel_); wrapper :107-122
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer owned by the caller (inputs, outputs and
+ *     workspace).  The library never allocates, frees or synchronises.
+ *   - Work is enqueued on `stream` (a hipStream_t; NULL = the default stream),
+ *     asynchronously and stream-ordered.
+ *   - Return value: M2_OK or a negative M2_ERR_* code; m2_last_error() returns a
+ *     thread-local message for the last failing call on this thread.
+ *   - Element strides are in ELEMENTS, the innermost dimension is contiguous
+ *     unless a stride for it is given.  x, B, C may be views into a packed
+ *     [x | B | C] or [z | x | B | C | dt] buffer (the reference packs them,
+ *     mamba2_kernel.py:71,109-115).
+ *   - Accumulation, cumulative sums, decays and SSM states are always fp32.
+ */
+#ifndef MAMBA2_HIP_H
+#define MAMBA2_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define M2_OK 0
+#define M2_ERR_SHAPE (-1)       /* a dimension is out of the supported set            */
+#define M2_ERR_DTYPE (-2)       /* unknown / unsupported element type                 */
+#define M2_ERR_ALIGN (-3)       /* pointer or stride not aligned for the vector path  */
+#define M2_ERR_WORKSPACE (-4)   /* workspace missing or too small                     */
+#define M2_ERR_LAUNCH (-5)      /* hipGetLastError() after a launch                   */
+#define M2_ERR_NULL (-6)        /* a required pointer is NULL                         */
+
+#define M2_F32 0
+#define M2_BF16 1
+
+#define M2_ACT_NONE 0
+#define M2_ACT_SILU 1
+#define M2_ACT_RELU 2
+
+#define M2_CHUNK 128            /* SSD chunk length (block_size = 128, mamba2_kernel.py:78) */
+
+/* ABI version of this header; bumped on any incompatible change. */
+int m2_abi_version(void);
+const char* m2_last_error(void);
+
+/* ------------------------------------------------------------------ conv1d
+ * y[b,t,c] = act(bias[c] + sum_{i<k} w[c,i] * x[b,t-(k-1)+i,c]),  x[t<0] = 0.
+ * Either layout is a stride choice: channels-last (b,l,C): stride_c == 1;
+ * channel-major (b,C,l) (ConvNKI's layout, conv1d_grouped.py:300-306): stride_l == 1.
+ * k in [1, 8].  w is (C, k) contiguous (the (C,1,k) parameter), bias (C) or NULL.
+ */
+typedef struct m2_conv1d_params {
+    const void* x; const void* w; const void* bias;   /* inputs                       */
+    const void* dy;                                    /* bwd only                     */
+    void* y;                                           /* fwd only                     */
+    void* dx; void* dw; void* db;                      /* bwd only; db may be NULL     */
+    void* workspace; size_t workspace_bytes;           /* bwd only                     */
+    int64_t batch, seqlen, channels; int32_t k;
+    int64_t x_stride_b, x_stride_l, x_stride_c;
+    int64_t y_stride_b, y_stride_l, y_stride_c;        /* y (fwd) / dy (bwd)           */
+    int64_t dx_stride_b, dx_stride_l, dx_stride_c;
+    int32_t dtype;                                     /* x, y, dy, dx                 */
+    int32_t param_dtype;                               /* w, bias, dw, db              */
+    int32_t activation;
+} m2_conv1d_params;
+
+int m2_conv1d_fwd(const m2_conv1d_params* p, void* stream);
+size_t m2_conv1d_bwd_workspace_bytes(int64_t batch, int64_t seqlen, int64_t channels, int32_t k);
+int m2_conv1d_bwd(const m2_conv1d_params* p, void* stream);
+
+/* ------------------------------------------------------------------ SSD scan
+ * dt (b,l,h), A (h) fp32, x (b,l,h,p), B,C (b,l,g,n), D (h) fp32 or NULL,
+ * initial_state / final_state (b,h,p,n) fp32 contiguous or NULL, y (b,l,h,p).
+ * Supported: p in {64,128}, n in {64,128}, h % g == 0, any l >= 0, any b >= 0.
+ * Backward additionally takes y (the forward output) and dy, and writes
+ * dx, ddt, dB, dC in the dtype of the matching input and dA (h), dD (h) in fp32,
+ * already summed over the batch (the reference sums them in its wrapper,
+ * mamba2_kernel.py:514).
+ */
+typedef struct m2_ssd_params {
+    const void* x; const void* dt; const float* A; const void* B; const void* C; const float* D;
+    const float* initial_state; float* final_state;
+    void* y;                                            /* fwd: out; bwd: in (saved forward output) */
+    /* backward only */
+    const void* dy; const float* d_final_state;
+    void* dx; void* ddt; float* dA; void* dB; void* dC; float* dD; float* d_initial_state;
+    void* workspace; size_t workspace_bytes;
+    int64_t batch, seqlen, nheads, headdim, dstate, ngroups;
+    int64_t x_stride_b, x_stride_l, x_stride_h;         /* x; innermost (p) contiguous  */
+    int64_t dt_stride_b, dt_stride_l;                   /* dt; innermost (h) contiguous */
+    int64_t B_stride_b, B_stride_l, B_stride_g;
+    int64_t C_stride_b, C_stride_l, C_stride_g;
+    int64_t y_stride_b, y_stride_l, y_stride_h;
+    int64_t dy_stride_b, dy_stride_l, dy_stride_h;
+    int64_t dx_stride_b, dx_stride_l, dx_stride_h;
+    int64_t ddt_stride_b, ddt_stride_l;
+    int64_t dB_stride_b, dB_stride_l, dB_stride_g;
+    int64_t dC_stride_b, dC_stride_l, dC_stride_g;
+    int32_t dtype;                                      /* x, B, C, y, dy, dx, dB, dC   */
+    int32_t dt_dtype;                                   /* dt, ddt                      */
+} m2_ssd_params;
+
+size_t m2_ssd_fwd_workspace_bytes(const m2_ssd_params* p);
+int m2_ssd_fwd(const m2_ssd_params* p, void* stream);
+size_t m2_ssd_bwd_workspace_bytes(const m2_ssd_params* p);
+int m2_ssd_bwd(const m2_ssd_params* p, void* stream);
+
+/* ------------------------------------------------------------------ decode step
+ * One token per batch row; conv_state (b,Cx,W) and S (b,h,p,n) fp32 are updated
+ * IN PLACE (the reference writes fresh copies and the caller re-binds them,
+ * mamba2_mixer.py:275-276).  W is k-1 or k columns.  SiLU is applied to all of
+ * [x | B | C] after the conv (mamba2_kernel_inference.py:14,69-90).
+ * workspace: b*Cx floats (activated conv output).
+ */
+typedef struct m2_decode_params {
+    const void* xBC; void* conv_state; const void* conv_w; const void* conv_b;
+    float* S; const void* dt; const float* A; const float* D; void* y;
+    void* workspace; size_t workspace_bytes;
+    int64_t batch, nheads, headdim, dstate, ngroups; int32_t k, W;
+    int64_t xBC_stride_b, dt_stride_b, y_stride_b;
+    int32_t dtype;                                      /* xBC, conv_state, dt, y       */
+    int32_t param_dtype;                                /* conv_w, conv_b               */
+    int32_t activation;
+} m2_decode_params;
+
+size_t m2_decode_workspace_bytes(int64_t batch, int64_t nheads, int64_t headdim, int64_t dstate, int64_t ngroups);
+int m2_decode_step(const m2_decode_params* p, void* stream);
+
+/* ------------------------------------------------------------------ self tests / probes
+ * m2_mfma_selftest: C (M x N fp32, row-major) = A (M x K) * Bt (N x K)^T through the same
+ * LDS-staged MFMA tile code the SSD kernels use.  M, N multiples of 128; K multiple of 32.
+ * m2_stream_copy: plain copy kernel of `bytes` bytes (multiple of 16), for calibrating
+ * bandwidth counters and the achievable-HBM figure.
+ */
+int m2_mfma_selftest(const void* A, const void* Bt, float* C, int64_t M, int64_t N, int64_t K, int32_t dtype, void* stream);
+int m2_stream_copy(const void* src, void* dst, size_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MAMBA2_HIP_H */

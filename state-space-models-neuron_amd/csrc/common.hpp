@@ -1,0 +1,98 @@
+// Shared device/host helpers for the gfx950 Mamba-2 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include <type_traits>
+
+#include "../../include/mamba2_hip.h"
+
+namespace m2 {
+
+// ----------------------------------------------------------------------------- errors
+void set_error(const char* fmt, ...);
+int fail(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+#define M2_REQUIRE(cond, code, ...) \
+    do { if (!(cond)) return ::m2::fail((code), __VA_ARGS__); } while (0)
+
+// ----------------------------------------------------------------------------- element types
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return (float)v; }
+
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return (bf16_t)v; }   // round-to-nearest-even
+
+template <typename T> struct VecTraits;
+template <> struct VecTraits<float> { static constexpr int kVec = 4; };     // 16-byte vectors
+template <> struct VecTraits<bf16_t> { static constexpr int kVec = 8; };
+
+// 16-byte vector of T, loaded/stored as one transaction; elements converted to fp32 on the fly.
+template <typename T> struct Vec16 {
+    static constexpr int N = VecTraits<T>::kVec;
+    T v[N];
+};
+template <typename T>
+__device__ __forceinline__ void load16(const T* __restrict__ p, float (&out)[VecTraits<T>::kVec]) {
+    constexpr int N = VecTraits<T>::kVec;
+    uint4 raw = *reinterpret_cast<const uint4*>(p);
+    const T* e = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+    for (int i = 0; i < N; ++i) out[i] = to_f32(e[i]);
+}
+template <typename T>
+__device__ __forceinline__ void store16(T* __restrict__ p, const float (&in)[VecTraits<T>::kVec]) {
+    constexpr int N = VecTraits<T>::kVec;
+    uint4 raw;
+    T* e = reinterpret_cast<T*>(&raw);
+#pragma unroll
+    for (int i = 0; i < N; ++i) e[i] = from_f32<T>(in[i]);
+    *reinterpret_cast<uint4*>(p) = raw;
+}
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + __expf(-z)); }
+// d/dz silu(z) = s * (1 + z * (1 - s)),  s = sigmoid(z)
+__device__ __forceinline__ float silu_grad_f(float z) {
+    float s = 1.0f / (1.0f + __expf(-z));
+    return s * (1.0f + z * (1.0f - s));
+}
+
+template <int ACT> __device__ __forceinline__ float act_f(float z) {
+    if (ACT == M2_ACT_SILU) return silu_f(z);
+    if (ACT == M2_ACT_RELU) return z > 0.f ? z : 0.f;
+    return z;
+}
+template <int ACT> __device__ __forceinline__ float act_grad_f(float z) {
+    if (ACT == M2_ACT_SILU) return silu_grad_f(z);
+    if (ACT == M2_ACT_RELU) return z > 0.f ? 1.f : 0.f;
+    return 1.f;
+}
+
+__device__ __forceinline__ float warp_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Dispatch a runtime dtype to a template type.
+#define M2_DISPATCH_DTYPE(dtype, T, ...)                                  \
+    do {                                                                  \
+        if ((dtype) == M2_F32) { using T = float; __VA_ARGS__; }          \
+        else if ((dtype) == M2_BF16) { using T = ::m2::bf16_t; __VA_ARGS__; } \
+        else return ::m2::fail(M2_ERR_DTYPE, "unsupported dtype %d", (int)(dtype)); \
+    } while (0)
+
+}  // namespace m2

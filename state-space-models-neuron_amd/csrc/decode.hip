@@ -1,0 +1,145 @@
+// Single-token recurrent decode step for gfx950.
+//
+// Replaces the reference's NKI kernel mamba_inference_kernel_ (mamba2/mamba2_kernel_inference.py:27-104):
+//   conv state shift + 1-token depthwise conv + SiLU on all of [x | B | C]     (:13-23)
+//   S' = S * exp(A dt) + (dt x) (x) B                                          (:81,95-97)
+//   y  = S' . C + D x                                                          (:101-102)
+//
+// The step is a pure streaming problem: per layer the fp32 state (b,h,p,n) is read once and written
+// once, in place (the reference writes fresh copies, doubling the footprint).  Two launches:
+//   decode_conv_kernel   one thread per (batch, channel): shifts the conv state in place and writes the
+//                        activated [x | B | C] row as fp32 into the workspace.  It must finish before any
+//                        state workgroup reads B/C, because every head of a group needs the same B/C
+//                        channels whose history is being overwritten in place.
+//   decode_ssm_kernel    one workgroup per (head, batch); a group of lanes owns one state row p and walks
+//                        n with 16-byte accesses, so a wave issues whole 128-byte-or-wider lines and every
+//                        state element is touched by exactly one thread (in-place update is race free).
+#include "common.hpp"
+
+namespace m2 {
+namespace {
+
+__device__ __forceinline__ float ld_any(const void* p, int dt, int64_t i) {
+    return dt == M2_F32 ? reinterpret_cast<const float*>(p)[i] : to_f32(reinterpret_cast<const bf16_t*>(p)[i]);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+decode_conv_kernel(const T* __restrict__ xBC, T* __restrict__ conv_state, const void* __restrict__ w, const void* __restrict__ bias,
+                   float* __restrict__ act, int64_t nb, int64_t Cx, int k, int W, int64_t xsb, int pd, int activation) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= nb * Cx) return;
+    const int64_t b = idx / Cx, c = idx % Cx;
+    T* cs = conv_state + idx * W;
+    float hist[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) hist[i] = 0.f;
+    T raw[8];
+    for (int i = 0; i < W; ++i) raw[i] = cs[i];
+    const T xin = xBC[b * xsb + c];
+    // taps: the last k-1 OLD columns, then the new input
+    float z = bias ? ld_any(bias, pd, c) : 0.f;
+    for (int i = 0; i < k - 1; ++i) z += ld_any(w, pd, c * k + i) * to_f32(raw[W - (k - 1) + i]);
+    z += ld_any(w, pd, c * k + (k - 1)) * to_f32(xin);
+    // shift left by one, append the input
+    for (int i = 0; i + 1 < W; ++i) cs[i] = raw[i + 1];
+    if (W > 0) cs[W - 1] = xin;
+    act[idx] = activation == M2_ACT_SILU ? silu_f(z) : (activation == M2_ACT_RELU ? (z > 0.f ? z : 0.f) : z);
+    (void)hist;
+}
+
+// VEC = 4: n % 4 == 0, float4 accesses; VEC = 1: any n.
+// GL lanes (a power of two <= 64) share one state row; rows per pass = 256 / GL.
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+decode_ssm_kernel(float* __restrict__ S, const float* __restrict__ act, const T* __restrict__ dt, const float* __restrict__ A,
+                  const float* __restrict__ D, T* __restrict__ y, int64_t nheads, int P, int N, int64_t ngroups, int64_t Cx,
+                  int64_t dtsb, int64_t ysb, int GL) {
+    const int tid = threadIdx.x;
+    const int64_t h = blockIdx.x, b = blockIdx.y;
+    const int64_t g = h / (nheads / ngroups);
+    const int64_t d_inner = nheads * P;
+    const float* xa = act + b * Cx + h * P;
+    const float* Ba = act + b * Cx + d_inner + g * N;
+    const float* Ca = act + b * Cx + d_inner + ngroups * N + g * N;
+    const float dtv = to_f32(dt[b * dtsb + h]);
+    const float dA = __expf(A[h] * dtv);
+    const float Dh = D ? D[h] : 0.f;
+    float* Sp = S + (b * nheads + h) * (int64_t)P * N;
+    const int sub = tid % GL, rowi = tid / GL, rows_per_pass = 256 / GL;
+    const int nv = N / VEC;
+    for (int p0 = 0; p0 < P; p0 += rows_per_pass) {
+        const int pp = p0 + rowi;
+        float part = 0.f, xv = 0.f;
+        if (pp < P) {
+            xv = xa[pp];
+            const float dx = dtv * xv;
+            for (int j = sub; j < nv; j += GL) {
+                if (VEC == 4) {
+                    floatx4 s = *reinterpret_cast<const floatx4*>(Sp + (int64_t)pp * N + j * 4);
+                    const floatx4 bv = *reinterpret_cast<const floatx4*>(Ba + j * 4);
+                    const floatx4 cv = *reinterpret_cast<const floatx4*>(Ca + j * 4);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) { s[q] = s[q] * dA + dx * bv[q]; part += s[q] * cv[q]; }
+                    *reinterpret_cast<floatx4*>(Sp + (int64_t)pp * N + j * 4) = s;
+                } else {
+                    float s = Sp[(int64_t)pp * N + j];
+                    s = s * dA + dx * Ba[j];
+                    part += s * Ca[j];
+                    Sp[(int64_t)pp * N + j] = s;
+                }
+            }
+        }
+        for (int off = GL >> 1; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+        if (pp < P && sub == 0) y[b * ysb + h * P + pp] = from_f32<T>(part + Dh * xv);
+    }
+}
+
+}  // namespace
+}  // namespace m2
+
+extern "C" size_t m2_decode_workspace_bytes(int64_t batch, int64_t nheads, int64_t headdim, int64_t dstate, int64_t ngroups) {
+    return (size_t)(batch * (nheads * headdim + 2 * ngroups * dstate)) * sizeof(float) + 16;
+}
+
+extern "C" int m2_decode_step(const m2_decode_params* p, void* stream) {
+    using namespace m2;
+    M2_REQUIRE(p, M2_ERR_NULL, "decode_step: params is NULL");
+    M2_REQUIRE(p->dtype == M2_F32 || p->dtype == M2_BF16, M2_ERR_DTYPE, "decode_step: bad dtype %d", p->dtype);
+    M2_REQUIRE(p->param_dtype == M2_F32 || p->param_dtype == M2_BF16, M2_ERR_DTYPE, "decode_step: bad param dtype %d", p->param_dtype);
+    M2_REQUIRE(p->batch >= 0 && p->nheads >= 0 && p->headdim >= 1 && p->dstate >= 1, M2_ERR_SHAPE, "decode_step: bad dimension");
+    M2_REQUIRE(p->ngroups >= 1 && p->nheads % p->ngroups == 0, M2_ERR_SHAPE, "decode_step: nheads %lld not divisible by ngroups %lld",
+               (long long)p->nheads, (long long)p->ngroups);
+    M2_REQUIRE(p->k >= 1 && p->k <= 8, M2_ERR_SHAPE, "decode_step: conv kernel size %d not in [1,8]", p->k);
+    M2_REQUIRE(p->W >= p->k - 1 && p->W <= 8, M2_ERR_SHAPE, "decode_step: conv state width %d must be in [k-1, 8]", p->W);
+    M2_REQUIRE(p->batch <= 65535, M2_ERR_SHAPE, "decode_step: batch exceeds the grid limit 65535");
+    if (p->batch == 0 || p->nheads == 0) return M2_OK;
+    M2_REQUIRE(p->xBC && p->conv_w && p->S && p->dt && p->A && p->y, M2_ERR_NULL, "decode_step: xBC, conv_w, S, dt, A, y are required");
+    M2_REQUIRE(p->W == 0 || p->conv_state, M2_ERR_NULL, "decode_step: conv_state is required");
+    const int64_t Cx = p->nheads * p->headdim + 2 * p->ngroups * p->dstate;
+    const size_t need = (size_t)(p->batch * Cx) * sizeof(float);
+    M2_REQUIRE(p->workspace && p->workspace_bytes >= need, M2_ERR_WORKSPACE, "decode_step: workspace %zu bytes < %zu needed",
+               p->workspace_bytes, need);
+    M2_REQUIRE(aligned16(p->workspace) && aligned16(p->S), M2_ERR_ALIGN, "decode_step: workspace and S must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    float* act = static_cast<float*>(p->workspace);
+    const int vec = (p->dstate % 4 == 0 && (p->nheads * p->headdim) % 4 == 0 && Cx % 4 == 0) ? 4 : 1;
+    int GL = 1;
+    while (GL < 64 && GL < p->dstate / vec) GL <<= 1;
+    M2_DISPATCH_DTYPE(p->dtype, T, {
+        decode_conv_kernel<T><<<(unsigned)ceil_div(p->batch * Cx, (int64_t)256), 256, 0, st>>>(
+            static_cast<const T*>(p->xBC), static_cast<T*>(p->conv_state), p->conv_w, p->conv_b, act, p->batch, Cx, p->k, p->W,
+            p->xBC_stride_b, p->param_dtype, p->activation);
+        int rc = check_launch("decode_conv_kernel");
+        if (rc) return rc;
+        dim3 grid((unsigned)p->nheads, (unsigned)p->batch);
+        if (vec == 4)
+            decode_ssm_kernel<T, 4><<<grid, 256, 0, st>>>(p->S, act, static_cast<const T*>(p->dt), p->A, p->D, static_cast<T*>(p->y),
+                                                          p->nheads, (int)p->headdim, (int)p->dstate, p->ngroups, Cx, p->dt_stride_b, p->y_stride_b, GL);
+        else
+            decode_ssm_kernel<T, 1><<<grid, 256, 0, st>>>(p->S, act, static_cast<const T*>(p->dt), p->A, p->D, static_cast<T*>(p->y),
+                                                          p->nheads, (int)p->headdim, (int)p->dstate, p->ngroups, Cx, p->dt_stride_b, p->y_stride_b, GL);
+        return check_launch("decode_ssm_kernel");
+    });
+    return M2_OK;
+}

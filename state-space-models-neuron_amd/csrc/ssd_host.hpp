@@ -1,0 +1,143 @@
+// Host-side helpers shared by the SSD forward and backward launchers.
+#pragma once
+#include "ssd_kernels.hpp"
+
+namespace m2 {
+
+// Workspace regions.  Forward uses G, local, prev, lam.  Backward additionally uses
+// sfinal (fp32 final state of the recomputed forward), dprev (gradient w.r.t. the state
+// leaving each chunk, operand type), dlam, per-(b,h,chunk) partials of dA and dD, and
+// per-(b,chunk,group,head-slice) fp32 partials of dB and dC.
+struct SsdWorkspace {
+    float* G = nullptr; float* local = nullptr; void* prev = nullptr; float* lam = nullptr;
+    float* sfinal = nullptr; void* dprev = nullptr; float* dlam = nullptr;
+    float* dAp = nullptr; float* dDp = nullptr; float* dBp = nullptr; float* dCp = nullptr;
+    int64_t nslices = 1, heads_per_slice = 1;
+    size_t bytes = 0;
+};
+
+// Heads of one group are processed by a workgroup in slices of `heads_per_slice`, so that the
+// group-level dB/dC reductions happen in registers; slices are chosen to give the GPU
+// at least ~768 workgroups when the shape allows.
+inline void ssd_bwd_slicing(const m2_ssd_params* p, int64_t* nslices, int64_t* hps) {
+    const int64_t nc = ceil_div(p->seqlen, (int64_t)kQ);
+    const int64_t hpg = p->nheads / p->ngroups;
+    const int64_t base = p->batch * nc * p->ngroups;
+    int64_t best = 1;
+    for (int64_t s = 1; s <= hpg; ++s) {
+        if (hpg % s) continue;
+        best = s;
+        if (base * s >= 768) break;
+    }
+    *nslices = best;
+    *hps = hpg / best;
+}
+
+inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd) {
+    const int64_t nc = ceil_div(p->seqlen, (int64_t)kQ);
+    const size_t esz = p->dtype == M2_F32 ? 4 : 2;
+    const size_t tiles = (size_t)p->batch * nc * p->nheads * p->headdim * p->dstate;
+    const size_t bhc = (size_t)p->batch * p->nheads * nc;
+    size_t off = 0;
+    SsdWorkspace w;
+    unsigned char* b8 = static_cast<unsigned char*>(base);
+    auto take = [&](size_t n) { unsigned char* r = b8 ? b8 + off : nullptr; off += align_up(n, 256); return r; };
+    w.G = reinterpret_cast<float*>(take((size_t)p->batch * nc * p->ngroups * kQ * kQ * 4));
+    w.local = reinterpret_cast<float*>(take(tiles * 4));
+    w.prev = take(tiles * esz);
+    w.lam = reinterpret_cast<float*>(take(bhc * 4));
+    if (bwd) {
+        ssd_bwd_slicing(p, &w.nslices, &w.heads_per_slice);
+        w.sfinal = reinterpret_cast<float*>(take((size_t)p->batch * p->nheads * p->headdim * p->dstate * 4));
+        w.dprev = take(tiles * esz);
+        w.dlam = reinterpret_cast<float*>(take(bhc * 4));
+        w.dAp = reinterpret_cast<float*>(take(bhc * 4));
+        w.dDp = reinterpret_cast<float*>(take(bhc * 4));
+        const size_t part = (size_t)p->batch * nc * p->ngroups * w.nslices * kQ * p->dstate * 4;
+        w.dBp = reinterpret_cast<float*>(take(part));
+        w.dCp = reinterpret_cast<float*>(take(part));
+    }
+    w.bytes = off + 256;
+    return w;
+}
+
+inline int ssd_check(const m2_ssd_params* p, const char* who) {
+    M2_REQUIRE(p, M2_ERR_NULL, "%s: params is NULL", who);
+    M2_REQUIRE(p->dtype == M2_F32 || p->dtype == M2_BF16, M2_ERR_DTYPE, "%s: bad dtype %d", who, p->dtype);
+    M2_REQUIRE(p->dt_dtype == M2_F32 || p->dt_dtype == p->dtype, M2_ERR_DTYPE,
+               "%s: dt dtype %d must be fp32 or the activation dtype", who, p->dt_dtype);
+    M2_REQUIRE(p->batch >= 0 && p->seqlen >= 0 && p->nheads >= 0, M2_ERR_SHAPE, "%s: negative dimension", who);
+    M2_REQUIRE(p->headdim == 64 || p->headdim == 128, M2_ERR_SHAPE, "%s: headdim %lld not in {64,128}", who, (long long)p->headdim);
+    M2_REQUIRE(p->dstate == 64 || p->dstate == 128, M2_ERR_SHAPE, "%s: dstate %lld not in {64,128}", who, (long long)p->dstate);
+    M2_REQUIRE(p->ngroups >= 1 && p->nheads % p->ngroups == 0, M2_ERR_SHAPE, "%s: nheads %lld not divisible by ngroups %lld", who,
+               (long long)p->nheads, (long long)p->ngroups);
+    M2_REQUIRE(p->batch <= 65535 && p->nheads <= 65535, M2_ERR_SHAPE, "%s: batch/nheads exceed the grid limit 65535", who);
+    const int V = p->dtype == M2_F32 ? 4 : 8;
+    M2_REQUIRE(p->x_stride_b % V == 0 && p->x_stride_l % V == 0 && p->x_stride_h % V == 0 &&
+               p->B_stride_b % V == 0 && p->B_stride_l % V == 0 && p->B_stride_g % V == 0 &&
+               p->C_stride_b % V == 0 && p->C_stride_l % V == 0 && p->C_stride_g % V == 0,
+               M2_ERR_ALIGN, "%s: x/B/C strides must be multiples of %d elements (16 bytes)", who, V);
+    M2_REQUIRE(aligned16(p->x) && aligned16(p->B) && aligned16(p->C), M2_ERR_ALIGN, "%s: x/B/C must be 16-byte aligned", who);
+    return M2_OK;
+}
+
+template <typename K>
+inline int allow_smem(K kernel, size_t bytes) {
+    if (bytes > 160 * 1024) return fail(M2_ERR_SHAPE, "kernel needs %zu bytes of LDS (> 160 KiB)", bytes);
+    if (bytes > 48 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)
+            return fail(M2_ERR_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS) failed: %s", bytes, hipGetErrorString(hipGetLastError()));
+    }
+    return M2_OK;
+}
+
+template <typename T, int P, int N>
+inline size_t state_smem() { return (3 * kQ + 4) * sizeof(float) + (size_t)(P + N) * lds_ld<T>(kQ) * sizeof(T); }
+template <typename T>
+inline size_t cb_smem() { return (size_t)2 * kQ * lds_ld<T>(64) * sizeof(T); }
+
+// G = C B^T, local chunk states, forward state scan.  Used by the forward and (recompute) by the backward.
+template <typename T, int P, int N>
+inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, float* final_out, hipStream_t st) {
+    const int64_t nc = ceil_div(p->seqlen, (int64_t)kQ);
+    const T* x = static_cast<const T*>(p->x);
+    const T* Bm = static_cast<const T*>(p->B);
+    const T* Cm = static_cast<const T*>(p->C);
+    const int dt_f32 = p->dt_dtype == M2_F32;
+    int rc;
+    {
+        auto k = cb_kernel<T, N>;
+        const size_t sm = cb_smem<T>();
+        if ((rc = allow_smem(k, sm))) return rc;
+        k<<<dim3((unsigned)nc, (unsigned)p->ngroups, (unsigned)p->batch), 256, sm, st>>>(
+            Bm, Cm, w.G, p->seqlen, p->ngroups, nc, p->B_stride_b, p->B_stride_l, p->B_stride_g,
+            p->C_stride_b, p->C_stride_l, p->C_stride_g);
+        if ((rc = check_launch("ssd cb_kernel"))) return rc;
+    }
+    {
+        auto k = chunk_state_kernel<T, P, N, false>;
+        const size_t sm = state_smem<T, P, N>();
+        if ((rc = allow_smem(k, sm))) return rc;
+        k<<<dim3((unsigned)nc, (unsigned)p->nheads, (unsigned)p->batch), 256, sm, st>>>(
+            x, p->dt, dt_f32, p->A, Bm, w.local, w.lam, p->seqlen, p->nheads, p->ngroups, nc,
+            p->x_stride_b, p->x_stride_l, p->x_stride_h, p->dt_stride_b, p->dt_stride_l,
+            p->B_stride_b, p->B_stride_l, p->B_stride_g);
+        if ((rc = check_launch("ssd chunk_state_kernel"))) return rc;
+    }
+    {
+        state_scan_kernel<T, P * N, false><<<dim3((unsigned)p->nheads, (unsigned)p->batch), 256, 0, st>>>(
+            w.local, w.lam, p->initial_state, static_cast<T*>(w.prev), final_out, nullptr, nullptr, nullptr, p->nheads, nc);
+        if ((rc = check_launch("ssd state_scan_kernel"))) return rc;
+    }
+    return M2_OK;
+}
+
+#define M2_DISPATCH_PN(p, P, N, ...)                                                     \
+    do {                                                                                 \
+        if ((p)->headdim == 64 && (p)->dstate == 64) { constexpr int P = 64, N = 64; __VA_ARGS__; }        \
+        else if ((p)->headdim == 64 && (p)->dstate == 128) { constexpr int P = 64, N = 128; __VA_ARGS__; } \
+        else if ((p)->headdim == 128 && (p)->dstate == 64) { constexpr int P = 128, N = 64; __VA_ARGS__; } \
+        else { constexpr int P = 128, N = 128; __VA_ARGS__; }                            \
+    } while (0)
+
+}  // namespace m2

@@ -1,0 +1,152 @@
+"""GPU: SSD chunked scan forward/backward parity against the fp64 CPU oracle (through the C ABI)."""
+import pytest
+import torch
+
+from conftest import rel_err, rel_rms_err
+from oracle.ssd import make_ssd_inputs, ssd_chunked_ref, ssd_grads_ref
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _tol(dtype):
+    return (1e-4, rel_err) if dtype == torch.float32 else (2e-2, rel_rms_err)
+
+
+def _dev(d):
+    return {k: v.to(DEV) for k, v in d.items()}
+
+
+def _f64(d):
+    return {k: v.double() for k, v in d.items()}
+
+
+CASES = [
+    # b, l, h, p, n, g
+    (1, 256, 8, 64, 64, 1),      # the fp32 correctness configuration
+    (2, 384, 4, 64, 128, 2),
+    (1, 200, 2, 128, 64, 1),     # ragged length, p = 128
+    (2, 128, 4, 128, 128, 4),
+    (1, 77, 2, 64, 128, 1),      # shorter than one chunk
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("b,l,h,p,n,g", CASES)
+def test_ssd_forward(dtype, b, l, h, p, n, g):
+    from mamba2.mamba2_kernel import mamba2_kernel
+    d = make_ssd_inputs(b, l, h, p, n, g, seed=l, dtype=dtype)
+    r = _f64(d)
+    y_ref, S_ref = ssd_chunked_ref(r["dt"], r["A"], r["X"], r["B"], r["C"], r["D"], chunk=64)
+    dd = _dev(d)
+    y, S = mamba2_kernel(dd["dt"], dd["A"], dd["X"], dd["B"], dd["C"], dd["D"], return_final_state=True)
+    tol, metric = _tol(dtype)
+    assert y.dtype == dtype and S.dtype == torch.float32
+    assert metric(y, y_ref) < tol, "y"
+    assert metric(S, S_ref) < tol, "final state"
+    y2 = mamba2_kernel(dd["dt"], dd["A"], dd["X"], dd["B"], dd["C"], dd["D"])
+    assert torch.equal(y2, y)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ssd_forward_initial_state_no_D_fp32_dt(dtype):
+    from mamba2.mamba2_kernel import mamba2_kernel
+    b, l, h, p, n, g = 2, 300, 4, 64, 64, 2
+    d = make_ssd_inputs(b, l, h, p, n, g, seed=9, dtype=dtype)
+    d["dt"] = d["dt"].float()                                  # fp32 dt next to bf16 activations
+    S0 = 0.1 * torch.randn(b, h, p, n, generator=torch.Generator().manual_seed(3))
+    r = _f64(d)
+    y_ref, S_ref = ssd_chunked_ref(r["dt"], r["A"], r["X"], r["B"], r["C"], None, initial_state=S0.double(), chunk=128)
+    dd = _dev(d)
+    y, S = mamba2_kernel(dd["dt"], dd["A"], dd["X"], dd["B"], dd["C"], None, initial_state=S0.to(DEV), return_final_state=True)
+    tol, metric = _tol(dtype)
+    assert metric(y, y_ref) < tol and metric(S, S_ref) < tol
+
+
+def test_ssd_packed_views():
+    # x, B, C as views into one packed [x | B | C] buffer, as the mixer passes them (mamba2_kernel.py:109-115,151)
+    from mamba2.mamba2_kernel import mamba2_kernel
+    b, l, h, p, n, g = 2, 256, 4, 64, 64, 2
+    d = make_ssd_inputs(b, l, h, p, n, g, seed=2, dtype=torch.bfloat16)
+    packed = torch.cat([d["X"].reshape(b, l, -1), d["B"].reshape(b, l, -1), d["C"].reshape(b, l, -1)], dim=-1).to(DEV)
+    X = packed[..., :h * p].unflatten(-1, (h, p))
+    Bm = packed[..., h * p:h * p + g * n].unflatten(-1, (g, n))
+    Cm = packed[..., h * p + g * n:].unflatten(-1, (g, n))
+    assert not X.is_contiguous()
+    dd = _dev(d)
+    y = mamba2_kernel(dd["dt"], dd["A"], X, Bm, Cm, dd["D"])
+    y2 = mamba2_kernel(dd["dt"], dd["A"], dd["X"], dd["B"], dd["C"], dd["D"])
+    assert torch.equal(y, y2)
+
+
+def test_ssd_special_cases():
+    from mamba2.mamba2_kernel import mamba2_kernel
+    b, l, h, p, n, g = 3, 256, 4, 64, 64, 1
+    d = _dev(make_ssd_inputs(1, l, h, p, n, g, seed=6))
+    rep = lambda t: t.repeat(b, *([1] * (t.dim() - 1)))
+    # batch-row consistency
+    y, S = mamba2_kernel(rep(d["dt"]), d["A"], rep(d["X"]), rep(d["B"]), rep(d["C"]), d["D"], return_final_state=True)
+    assert torch.equal(y[0], y[1]) and torch.equal(y[0], y[2]) and torch.equal(S[0], S[2])
+    # zero in -> zero out;  B = C = 0 -> y = D x
+    z = torch.zeros_like(d["X"])
+    y, S = mamba2_kernel(d["dt"], d["A"], z, d["B"], d["C"], d["D"], return_final_state=True)
+    assert y.abs().max() == 0 and S.abs().max() == 0
+    zb = torch.zeros_like(d["B"])
+    y = mamba2_kernel(d["dt"], d["A"], d["X"], zb, zb, d["D"])
+    assert torch.allclose(y, d["D"][None, None, :, None] * d["X"], atol=1e-6)
+    # empty
+    y, S = mamba2_kernel(d["dt"][:, :0], d["A"], d["X"][:, :0], d["B"][:, :0], d["C"][:, :0], d["D"], return_final_state=True)
+    assert y.shape == (1, 0, h, p) and S.abs().max() == 0
+
+
+def test_ssd_rejects_unsupported():
+    from mamba2.mamba2_kernel import mamba2_kernel
+    d = _dev(make_ssd_inputs(1, 128, 2, 32, 64, 1, seed=0))
+    with pytest.raises(ValueError, match="headdim"):
+        mamba2_kernel(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"])
+    d = make_ssd_inputs(1, 128, 2, 64, 64, 1, seed=0)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        mamba2_kernel(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("b,l,h,p,n,g", CASES)
+def test_ssd_backward(dtype, b, l, h, p, n, g):
+    from mamba2.mamba2_kernel import mamba2_kernel
+    d = make_ssd_inputs(b, l, h, p, n, g, seed=l + 1, dtype=dtype)
+    r = _f64(d)
+    ref = ssd_grads_ref(r["dt"], r["A"], r["X"], r["B"], r["C"], r["D"], r["dy"], chunk=64)
+    dd = _dev(d)
+    leaves = {k: dd[k].clone().requires_grad_(True) for k in ("dt", "A", "X", "B", "C", "D")}
+    y = mamba2_kernel(leaves["dt"], leaves["A"], leaves["X"], leaves["B"], leaves["C"], leaves["D"])
+    y.backward(dd["dy"])
+    tol, metric = _tol(dtype)
+    for name, key in (("dX", "X"), ("ddt", "dt"), ("dA", "A"), ("dB", "B"), ("dC", "C"), ("dD", "D")):
+        e = metric(leaves[key].grad, ref[name])
+        assert e < tol, f"{name}: {e}"
+    assert leaves["X"].grad.dtype == dtype and leaves["dt"].grad.dtype == dtype and leaves["A"].grad.dtype == torch.float32
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ssd_backward_states(dtype):
+    # gradient through the final state and into the initial state
+    from mamba2.mamba2_kernel import mamba2_kernel
+    b, l, h, p, n, g = 2, 300, 4, 64, 64, 2
+    d = make_ssd_inputs(b, l, h, p, n, g, seed=12, dtype=dtype)
+    gen = torch.Generator().manual_seed(4)
+    S0 = 0.1 * torch.randn(b, h, p, n, generator=gen)
+    dS = torch.randn(b, h, p, n, generator=gen)
+    r = _f64(d)
+    ref = ssd_grads_ref(r["dt"], r["A"], r["X"], r["B"], r["C"], r["D"], r["dy"], initial_state=S0.double(),
+                        d_final_state=dS.double(), chunk=128)
+    dd = _dev(d)
+    leaves = {k: dd[k].clone().requires_grad_(True) for k in ("dt", "A", "X", "B", "C", "D")}
+    S0d = S0.to(DEV).requires_grad_(True)
+    y, S = mamba2_kernel(leaves["dt"], leaves["A"], leaves["X"], leaves["B"], leaves["C"], leaves["D"], initial_state=S0d,
+                         return_final_state=True)
+    torch.autograd.backward([y, S], [dd["dy"], dS.to(DEV)])
+    tol, metric = _tol(dtype)
+    for name, key in (("dX", "X"), ("ddt", "dt"), ("dA", "A"), ("dB", "B"), ("dC", "C"), ("dD", "D")):
+        e = metric(leaves[key].grad, ref[name])
+        assert e < tol, f"{name}: {e}"
+    assert metric(S0d.grad, ref["dinitial_state"]) < tol
