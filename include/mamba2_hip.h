@@ -87,7 +87,7 @@ int m2_conv1d_bwd(const m2_conv1d_params* p, void* stream);
  * dt (b,l,h), A (h) fp32, x (b,l,h,p), B,C (b,l,g,n), D (h) fp32 or NULL,
  * initial_state / final_state (b,h,p,n) fp32 contiguous or NULL, y (b,l,h,p).
  * Supported: p in {64,128}, n in {64,128}, h % g == 0, any l >= 0, any b >= 0.
- * Backward additionally takes y (the forward output) and dy, and writes
+ * Backward takes the same inputs plus dy (it recomputes per chunk; y is unused) and writes
  * dx, ddt, dB, dC in the dtype of the matching input and dA (h), dD (h) in fp32,
  * already summed over the batch (the reference sums them in its wrapper,
  * mamba2_kernel.py:514).
@@ -95,7 +95,7 @@ int m2_conv1d_bwd(const m2_conv1d_params* p, void* stream);
 typedef struct m2_ssd_params {
     const void* x; const void* dt; const float* A; const void* B; const void* C; const float* D;
     const float* initial_state; float* final_state;
-    void* y;                                            /* fwd: out; bwd: in (saved forward output) */
+    void* y;                                            /* fwd: out; unused by bwd      */
     /* backward only */
     const void* dy; const float* d_final_state;
     void* dx; void* ddt; float* dA; void* dB; void* dC; float* dD; float* d_initial_state;

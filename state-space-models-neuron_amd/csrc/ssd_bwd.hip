@@ -11,20 +11,23 @@
 //   dG[i][j] = sum_h e^{l_i-l_j} dt_j (dy_i . x_j)           (i >= j, summed over the heads of a group)
 //   dC_i = sum_j dG[i][j] B_j + sum_h e^{l_i} dy_i^T S_prev
 //   dB_j = sum_i dG[i][j] C_i + sum_h dt_j e^{Lam-l_j} x_j^T dS
-//   dl_i = dy_i . (y_i - D x_i) - xd_i . dxd_i               (row role minus column role of l_i)
+//   dl_i = sum_n (C_i o dC_i^h - B_i o dB_i^h)               (row role minus column role of l_i, per head;
+//                                                             the reference's C o dC - B o dB, :401,456)
+//        = rowsum_i(dG^h o G) - colsum_i(dG^h o G) + C_i . dCoff_i^h - B_i . dBoff_i^h
 //   da_j = sum_{i>=j, same chunk} dl_i + <dS, S_new>         ddt_j = A da_j + dxd_j . x_j
 //   dA   = sum_j da_j dt_j                                   dD = sum dy . x
-// The identity for dl uses the forward output y, so the backward takes y as an input instead of
-// recomputing it; the reference gets the same quantity from C o dC - B o dB (:401,456).
-// <dS, S_new> is exact per chunk, so rounding does not accumulate along the sequence as it would
-// with a global reverse cumulative sum (:459-461).
+// Row sums and column sums are taken from the SAME fp32 tile dG^h o G, so pairs (i, j) that both lie
+// in a suffix cancel exactly and only pairs straddling the position contribute, as in exact
+// arithmetic.  (Forming dl from dy . (y - D x) with the stored bf16 y loses everything to
+// cancellation once D x dominates y.)  <dS, S_new> is exact per chunk, so rounding does not
+// accumulate along the sequence as it would with a global reverse cumulative sum (:459-461).
 //
 // Launch sequence:
 //   cb_kernel, chunk_state_kernel, state_scan_kernel          recompute G, S_prev, final state
 //   chunk_state_kernel<DSTATE>                                local dS contributions  e^{l} dy^T C
 //   state_scan_kernel<REVERSE>                                dS per chunk, <dS, S_new>, d initial state
+//   group_grad_kernel      per (b, chunk, group, head slice)  partial dB, dC (heads reduced in registers), dl per head
 //   dx_kernel              per (b, chunk, head)               dx, ddt, partial dA, dD
-//   group_grad_kernel      per (b, chunk, group, head slice)  partial dB, dC (heads reduced in registers)
 //   bc_reduce_kernel, ad_reduce_kernel                        sum the partials (fixed order, no atomics)
 #include "ssd_host.hpp"
 
@@ -43,11 +46,11 @@ template <typename T, int P, int N>
 __global__ void __launch_bounds__(256)
 dx_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f32, const float* __restrict__ A,
           const T* __restrict__ Bm, const float* __restrict__ D, const float* __restrict__ G,
-          const T* __restrict__ Y, const T* __restrict__ dY, const T* __restrict__ dprev, const float* __restrict__ dlam,
+          const float* __restrict__ dl, const T* __restrict__ dY, const T* __restrict__ dprev, const float* __restrict__ dlam,
           T* __restrict__ dX, void* __restrict__ ddt, float* __restrict__ dAp, float* __restrict__ dDp,
           int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks,
           int64_t Xsb, int64_t Xsl, int64_t Xsh, int64_t dtsb, int64_t dtsl,
-          int64_t Bsb, int64_t Bsl, int64_t Bsg, int64_t Ysb, int64_t Ysl, int64_t Ysh,
+          int64_t Bsb, int64_t Bsl, int64_t Bsg,
           int64_t dYsb, int64_t dYsl, int64_t dYsh, int64_t dXsb, int64_t dXsl, int64_t dXsh,
           int64_t ddtsb, int64_t ddtsl) {
     constexpr int LDN = lds_ld<T>(N);
@@ -113,32 +116,27 @@ dx_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f32, cons
     // ---- epilogue
     const float Dh = D ? D[h] : 0.f;
     const T* Xp = X + b * Xsb + t0 * Xsl + h * Xsh;
-    const T* Yp = Y + b * Ysb + t0 * Ysl + h * Ysh;
     T* dXp = dX + b * dXsb + t0 * dXsl + h * dXsh;
     float dD_loc = 0.f;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
         const int row = wave * 32 + acc_row(lane, v);
-        float ew = 0.f, edir = 0.f;
+        float edir = 0.f;
         if (row < valid) {
             const float dtj = s_dt[row];
 #pragma unroll
             for (int j = 0; j < BN; ++j) {
                 const int col = j * 32 + acc_col(lane);
                 const float xv = to_f32(Xp[(int64_t)row * Xsl + col]);
-                const float yv = to_f32(Yp[(int64_t)row * Ysl + col]);
                 const float gy = to_f32(sdYt[col * LDQ + row]);
                 const float dxd = acc[0][j][v];
                 dXp[(int64_t)row * dXsl + col] = from_f32<T>(dtj * dxd + Dh * gy);
-                const float dxdx = dxd * xv;
-                edir += dxdx;
-                ew += gy * (yv - Dh * xv) - dtj * dxdx;
+                edir += dxd * xv;
                 dD_loc += gy * xv;
             }
         }
-        ew = half_wave_sum(ew);
         edir = half_wave_sum(edir);
-        if ((lane & 31) == 0) { s_w[row] = ew; s_dir[row] = edir; }
+        if ((lane & 31) == 0) s_dir[row] = edir;
     }
     dD_loc = warp_sum(dD_loc);
     if (lane == 0) s_red[wave] = dD_loc;
@@ -148,7 +146,7 @@ dx_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f32, cons
     float da_dt = 0.f;
     if (tid < kQ) {
         const int j = kQ - 1 - tid;                // thread t scans token Q-1-t: prefix over t == suffix over j
-        float s = s_w[j];
+        float s = dl[((b * nheads + h) * nchunks + c) * kQ + j];
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
             const float nb = __shfl_up(s, off, 64);
@@ -188,8 +186,8 @@ template <typename T, int P, int N>
 __global__ void __launch_bounds__(512)
 group_grad_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f32, const float* __restrict__ A,
                   const T* __restrict__ Bm, const T* __restrict__ Cm, const T* __restrict__ dY,
-                  const T* __restrict__ Sprev, const T* __restrict__ dprev,
-                  float* __restrict__ dBp, float* __restrict__ dCp,
+                  const T* __restrict__ Sprev, const T* __restrict__ dprev, const float* __restrict__ G,
+                  float* __restrict__ dBp, float* __restrict__ dCp, float* __restrict__ dl,
                   int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks, int64_t nslices, int64_t hps,
                   int64_t Xsb, int64_t Xsl, int64_t Xsh, int64_t dtsb, int64_t dtsl,
                   int64_t Bsb, int64_t Bsl, int64_t Bsg, int64_t Csb, int64_t Csl, int64_t Csg,
@@ -206,7 +204,11 @@ group_grad_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f
     float* s_e = s_dt + kQ;                        // e^{l_i}
     float* s_d = s_e + kQ;                         // dt_j e^{Lam - l_j}
     float* s_tmp = s_d + kQ;                       // 4 floats
-    T* buf = reinterpret_cast<T*>(s_tmp + 4);
+    float* s_rs = s_tmp + 4;                       // [2][kQ] row sums of dG^h o G   (one slot per column half)
+    float* s_cs = s_rs + 2 * kQ;                   // [4][kQ] column sums of dG^h o G (one slot per row block)
+    float* s_rc = s_cs + 4 * kQ;                   // [2][kQ] C_i . dCoff_i^h
+    float* s_rb = s_rc + 2 * kQ;                   // [2][kQ] B_j . dBoff_j^h
+    T* buf = reinterpret_cast<T*>(s_rb + 2 * kQ);
     T* sA = buf;                                   // first tile  [kQ][LDP]  (or [kQ][LDQ] in the final steps)
     T* sT = buf + kQ * LDP;                        // second tile [kQ or N][LDP]
     T* sA2 = buf;                                  // final: [kQ][LDQ]
@@ -237,9 +239,14 @@ group_grad_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f
         stage_rows<T, kQ, P, 512, false>(sA, LDP, dYp, dYsl, valid, nullptr, tid);
         stage_rows<T, kQ, P, 512, false>(sT, LDP, Xp, Xsl, valid, nullptr, tid);
         __syncthreads();
+        const float* Gp = G + ((b * nchunks + c) * ngroups + g) * (int64_t)(kQ * kQ);
         {
             floatx16 pa[1][2];
             acc_zero(pa);
+            float rsum[16], csum[2];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) rsum[v] = 0.f;
+            csum[0] = csum[1] = 0.f;
             if (cb0 <= rb) {
                 wave_mma<1, 2>(pa, sA + rb * 32 * LDP, LDP, sT + cb0 * 32 * LDP, LDP, 0, P);
 #pragma unroll
@@ -250,55 +257,133 @@ group_grad_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int i = rb * 32 + acc_row(lane, v);
-                        if (i >= j) dG[0][jb][v] += __expf(s_l[i] - lj) * dtj * pa[0][jb][v];
+                        if (i >= j) {
+                            const float dgh = __expf(s_l[i] - lj) * dtj * pa[0][jb][v];
+                            dG[0][jb][v] += dgh;
+                            const float pr = dgh * Gp[i * kQ + j];
+                            rsum[v] += pr;
+                            csum[jb] += pr;
+                        }
                     }
                 }
+            }
+            // row sums: over the 32 lanes of a half wave (columns) -> slot (wave & 1) of row i
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float r = half_wave_sum(rsum[v]);
+                if ((lane & 31) == 0) s_rs[(wave & 1) * kQ + rb * 32 + acc_row(lane, v)] = r;
+            }
+            // column sums: over this lane's 16 rows, then the other half wave -> slot rb of column j
+#pragma unroll
+            for (int jb = 0; jb < 2; ++jb) {
+                const float cs = csum[jb] + __shfl_xor(csum[jb], 32, 64);
+                if (lane < 32) s_cs[rb * kQ + (cb0 + jb) * 32 + lane] = cs;
             }
         }
         __syncthreads();
 
-        // ---- B: dC[i][n] += sum_p (e^{l_i} dy[i][p]) S_prev[p][n]
-        stage_rows<T, kQ, P, 512, true>(sA, LDP, dYp, dYsl, valid, s_e, tid);
+        // ---- B: dC[i][n] += e^{l_i} sum_p dy[i][p] S_prev[p][n]     (dy tile still in sA; row scale applied in fp32)
         stage_transposed<T, P, N, 512, false>(sT, LDP, Sprev + tile, N, P, nullptr, tid);
         __syncthreads();
-        wave_mma<1, NB>(dC, sA + rb * 32 * LDP, LDP, sT + nb0 * 32 * LDP, LDP, 0, P);
+        {
+            floatx16 tc[1][NB];
+            acc_zero(tc);
+            wave_mma<1, NB>(tc, sA + rb * 32 * LDP, LDP, sT + nb0 * 32 * LDP, LDP, 0, P);
+            const T* Cg = Cm + b * Csb + t0 * Csl + g * Csg;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int i = rb * 32 + acc_row(lane, v);
+                const float sc = s_e[i];
+                float r = 0.f;
+#pragma unroll
+                for (int jn = 0; jn < NB; ++jn) {
+                    const float t = tc[0][jn][v] * sc;
+                    dC[0][jn][v] += t;
+                    if (i < valid) r += t * to_f32(Cg[(int64_t)i * Csl + (nb0 + jn) * 32 + acc_col(lane)]);
+                }
+                r = half_wave_sum(r);
+                if ((lane & 31) == 0) s_rc[(wave & 1) * kQ + i] = r;
+            }
+        }
         __syncthreads();
 
-        // ---- C: dB[j][n] += sum_p (dt_j e^{Lam-l_j} x[j][p]) dS[p][n]
-        stage_rows<T, kQ, P, 512, true>(sA, LDP, Xp, Xsl, valid, s_d, tid);
+        // ---- C: dB[j][n] += dt_j e^{Lam-l_j} sum_p x[j][p] dS[p][n]
+        stage_rows<T, kQ, P, 512, false>(sA, LDP, Xp, Xsl, valid, nullptr, tid);
         stage_transposed<T, P, N, 512, false>(sT, LDP, dprev + tile, N, P, nullptr, tid);
         __syncthreads();
-        wave_mma<1, NB>(dB, sA + rb * 32 * LDP, LDP, sT + nb0 * 32 * LDP, LDP, 0, P);
+        {
+            floatx16 tb[1][NB];
+            acc_zero(tb);
+            wave_mma<1, NB>(tb, sA + rb * 32 * LDP, LDP, sT + nb0 * 32 * LDP, LDP, 0, P);
+            const T* Bg = Bm + b * Bsb + t0 * Bsl + g * Bsg;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int j = rb * 32 + acc_row(lane, v);
+                const float sc = s_d[j];
+                float r = 0.f;
+#pragma unroll
+                for (int jn = 0; jn < NB; ++jn) {
+                    const float t = tb[0][jn][v] * sc;
+                    dB[0][jn][v] += t;
+                    if (j < valid) r += t * to_f32(Bg[(int64_t)j * Bsl + (nb0 + jn) * 32 + acc_col(lane)]);
+                }
+                r = half_wave_sum(r);
+                if ((lane & 31) == 0) s_rb[(wave & 1) * kQ + j] = r;
+            }
+        }
         __syncthreads();
+        // dl_t for this head: row role minus column role
+        if (tid < kQ) {
+            const float rs = s_rs[tid] + s_rs[kQ + tid];
+            const float cs = s_cs[tid] + s_cs[kQ + tid] + s_cs[2 * kQ + tid] + s_cs[3 * kQ + tid];
+            const float rc = s_rc[tid] + s_rc[kQ + tid];
+            const float rbv = s_rb[tid] + s_rb[kQ + tid];
+            dl[((b * nheads + h) * nchunks + c) * kQ + tid] = rs - cs + rc - rbv;
+        }
     }
 
     const T* Bp = Bm + b * Bsb + t0 * Bsl + g * Bsg;
     const T* Cp = Cm + b * Csb + t0 * Csl + g * Csg;
 
+    // The head-summed dG is rounded to the operand type only here.  For bf16 it is split into
+    // hi + lo (two MFMA passes) so that the group-level contractions see it at ~2^-17 relative.
+    constexpr int NPASS = sizeof(T) == 2 ? 2 : 1;
+
     // ---- F1: dC[i][n] += sum_{j<=i} dG[i][j] B[j][n]
-#pragma unroll
-    for (int jb = 0; jb < 2; ++jb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int i = rb * 32 + acc_row(lane, v), j = (cb0 + jb) * 32 + acc_col(lane);
-            sA2[i * LDQ + j] = from_f32<T>(dG[0][jb][v]);
-        }
     stage_transposed<T, kQ, N, 512, false>(sT2, LDQ, Bp, Bsl, valid, nullptr, tid);
-    __syncthreads();
-    wave_mma<1, NB>(dC, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, 0, (rb + 1) * 32);
-    __syncthreads();
+#pragma unroll
+    for (int pass = 0; pass < NPASS; ++pass) {
+#pragma unroll
+        for (int jb = 0; jb < 2; ++jb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int i = rb * 32 + acc_row(lane, v), j = (cb0 + jb) * 32 + acc_col(lane);
+                const float full = dG[0][jb][v];
+                const T hi = from_f32<T>(full);
+                sA2[i * LDQ + j] = pass == 0 ? hi : from_f32<T>(full - to_f32(hi));
+            }
+        __syncthreads();
+        wave_mma<1, NB>(dC, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, 0, (rb + 1) * 32);
+        __syncthreads();
+    }
 
     // ---- F2: dB[j][n] += sum_{i>=j} dG[i][j] C[i][n]
-#pragma unroll
-    for (int jb = 0; jb < 2; ++jb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int i = rb * 32 + acc_row(lane, v), j = (cb0 + jb) * 32 + acc_col(lane);
-            sA2[j * LDQ + i] = from_f32<T>(dG[0][jb][v]);
-        }
     stage_transposed<T, kQ, N, 512, false>(sT2, LDQ, Cp, Csl, valid, nullptr, tid);
-    __syncthreads();
-    wave_mma<1, NB>(dB, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, rb * 32, kQ);
+#pragma unroll
+    for (int pass = 0; pass < NPASS; ++pass) {
+#pragma unroll
+        for (int jb = 0; jb < 2; ++jb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int i = rb * 32 + acc_row(lane, v), j = (cb0 + jb) * 32 + acc_col(lane);
+                const float full = dG[0][jb][v];
+                const T hi = from_f32<T>(full);
+                sA2[j * LDQ + i] = pass == 0 ? hi : from_f32<T>(full - to_f32(hi));
+            }
+        __syncthreads();
+        wave_mma<1, NB>(dB, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, rb * 32, kQ);
+        __syncthreads();
+    }
 
     // ---- store partials [b][c][g][slice][Q][N]
     const int64_t pt = (((b * nchunks + c) * ngroups + g) * nslices + slice) * (int64_t)(kQ * N);
@@ -380,7 +465,7 @@ size_t gg_smem() {
     size_t a = (size_t)2 * kQ * lds_ld<T>(P), b = (size_t)(kQ + N) * lds_ld<T>(kQ), c = (size_t)(kQ + N) * lds_ld<T>(P);
     size_t m = a > b ? a : b;
     m = m > c ? m : c;
-    return (4 * kQ + 4) * sizeof(float) + m * sizeof(T);
+    return (14 * kQ + 4) * sizeof(float) + m * sizeof(T);
 }
 
 template <typename T, int P, int N>
@@ -411,30 +496,30 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         if ((rc = check_launch("ssd state_scan_kernel<reverse>"))) return rc;
     }
     {
-        auto k = dx_kernel<T, P, N>;
-        const size_t sm = dx_smem<T, P, N>();
-        if ((rc = allow_smem(k, sm))) return rc;
-        k<<<dim3((unsigned)nc, (unsigned)p->nheads, (unsigned)p->batch), 256, sm, st>>>(
-            x, p->dt, dt_f32, p->A, Bm, p->D, w.G, static_cast<const T*>(p->y), dy, static_cast<const T*>(w.dprev), w.dlam,
-            static_cast<T*>(p->dx), p->ddt, w.dAp, w.dDp, p->seqlen, p->nheads, p->ngroups, nc,
-            p->x_stride_b, p->x_stride_l, p->x_stride_h, p->dt_stride_b, p->dt_stride_l,
-            p->B_stride_b, p->B_stride_l, p->B_stride_g, p->y_stride_b, p->y_stride_l, p->y_stride_h,
-            p->dy_stride_b, p->dy_stride_l, p->dy_stride_h, p->dx_stride_b, p->dx_stride_l, p->dx_stride_h,
-            p->ddt_stride_b, p->ddt_stride_l);
-        if ((rc = check_launch("ssd dx_kernel"))) return rc;
-    }
-    {
         auto k = group_grad_kernel<T, P, N>;
         const size_t sm = gg_smem<T, P, N>();
         if ((rc = allow_smem(k, sm))) return rc;
         M2_REQUIRE(p->ngroups * w.nslices <= 65535, M2_ERR_SHAPE, "ssd_bwd: too many group slices");
         k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * w.nslices), (unsigned)p->batch), 512, sm, st>>>(
-            x, p->dt, dt_f32, p->A, Bm, Cm, dy, static_cast<const T*>(w.prev), static_cast<const T*>(w.dprev), w.dBp, w.dCp,
+            x, p->dt, dt_f32, p->A, Bm, Cm, dy, static_cast<const T*>(w.prev), static_cast<const T*>(w.dprev), w.G, w.dBp, w.dCp, w.dl,
             p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice,
             p->x_stride_b, p->x_stride_l, p->x_stride_h, p->dt_stride_b, p->dt_stride_l,
             p->B_stride_b, p->B_stride_l, p->B_stride_g, p->C_stride_b, p->C_stride_l, p->C_stride_g,
             p->dy_stride_b, p->dy_stride_l, p->dy_stride_h);
         if ((rc = check_launch("ssd group_grad_kernel"))) return rc;
+    }
+    {
+        auto k = dx_kernel<T, P, N>;
+        const size_t sm = dx_smem<T, P, N>();
+        if ((rc = allow_smem(k, sm))) return rc;
+        k<<<dim3((unsigned)nc, (unsigned)p->nheads, (unsigned)p->batch), 256, sm, st>>>(
+            x, p->dt, dt_f32, p->A, Bm, p->D, w.G, w.dl, dy, static_cast<const T*>(w.dprev), w.dlam,
+            static_cast<T*>(p->dx), p->ddt, w.dAp, w.dDp, p->seqlen, p->nheads, p->ngroups, nc,
+            p->x_stride_b, p->x_stride_l, p->x_stride_h, p->dt_stride_b, p->dt_stride_l,
+            p->B_stride_b, p->B_stride_l, p->B_stride_g,
+            p->dy_stride_b, p->dy_stride_l, p->dy_stride_h, p->dx_stride_b, p->dx_stride_l, p->dx_stride_h,
+            p->ddt_stride_b, p->ddt_stride_l);
+        if ((rc = check_launch("ssd dx_kernel"))) return rc;
     }
     {
         const int64_t total = p->batch * p->seqlen * p->ngroups * (N / 4);
@@ -474,7 +559,7 @@ extern "C" int m2_ssd_bwd(const m2_ssd_params* p, void* stream) {
         }
         return check_launch("ssd_bwd (empty)");
     }
-    M2_REQUIRE(p->x && p->dt && p->A && p->B && p->C && p->y && p->dy, M2_ERR_NULL, "ssd_bwd: x, dt, A, B, C, y, dy are required");
+    M2_REQUIRE(p->x && p->dt && p->A && p->B && p->C && p->dy, M2_ERR_NULL, "ssd_bwd: x, dt, A, B, C, dy are required");
     M2_REQUIRE(p->dx && p->ddt && p->dB && p->dC, M2_ERR_NULL, "ssd_bwd: dx, ddt, dB, dC are required");
     const int V = p->dtype == M2_F32 ? 4 : 8;
     M2_REQUIRE(p->dy_stride_b % V == 0 && p->dy_stride_l % V == 0 && p->dy_stride_h % V == 0 && aligned16(p->dy), M2_ERR_ALIGN,

@@ -6,12 +6,13 @@ namespace m2 {
 
 // Workspace regions.  Forward uses G, local, prev, lam.  Backward additionally uses
 // sfinal (fp32 final state of the recomputed forward), dprev (gradient w.r.t. the state
-// leaving each chunk, operand type), dlam, per-(b,h,chunk) partials of dA and dD, and
+// leaving each chunk, operand type), dlam, dl (per-token gradient of the in-chunk cumulative
+// sum, per head), per-(b,h,chunk) partials of dA and dD, and
 // per-(b,chunk,group,head-slice) fp32 partials of dB and dC.
 struct SsdWorkspace {
     float* G = nullptr; float* local = nullptr; void* prev = nullptr; float* lam = nullptr;
     float* sfinal = nullptr; void* dprev = nullptr; float* dlam = nullptr;
-    float* dAp = nullptr; float* dDp = nullptr; float* dBp = nullptr; float* dCp = nullptr;
+    float* dAp = nullptr; float* dDp = nullptr; float* dBp = nullptr; float* dCp = nullptr; float* dl = nullptr;
     int64_t nslices = 1, heads_per_slice = 1;
     size_t bytes = 0;
 };
@@ -53,6 +54,7 @@ inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd) {
         w.dlam = reinterpret_cast<float*>(take(bhc * 4));
         w.dAp = reinterpret_cast<float*>(take(bhc * 4));
         w.dDp = reinterpret_cast<float*>(take(bhc * 4));
+        w.dl = reinterpret_cast<float*>(take(bhc * kQ * 4));
         const size_t part = (size_t)p->batch * nc * p->ngroups * w.nslices * kQ * p->dstate * 4;
         w.dBp = reinterpret_cast<float*>(take(part));
         w.dCp = reinterpret_cast<float*>(take(part));

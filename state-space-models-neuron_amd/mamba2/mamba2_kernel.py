@@ -81,7 +81,7 @@ def ssd_forward(dt, A, X, B, C, D=None, initial_state=None, want_final_state=Fal
     return Y, S
 
 
-def ssd_backward(dt, A, X, B, C, D, Y, dY, initial_state=None, d_final_state=None, want_dinitial=False,
+def ssd_backward(dt, A, X, B, C, D, dY, initial_state=None, d_final_state=None, want_dinitial=False,
                  out_dX=None, out_dB=None, out_dC=None):
     """Raw backward through the C ABI.
     Returns (ddt, dA fp32 (h), dX, dB, dC, dD fp32 (h) or None, d_initial_state or None).
@@ -109,9 +109,8 @@ def ssd_backward(dt, A, X, B, C, D, Y, dY, initial_state=None, d_final_state=Non
     dS0 = torch.empty((b, h, hd, n), dtype=torch.float32, device=dev) if want_dinitial else None
     p = SsdParams()
     _fill_common(p, dt, A32, X, B, C, D32)
-    p.initial_state, p.y, p.dy, p.d_final_state = ptr(S0), ptr(Y), ptr(dY), ptr(dSf)
+    p.initial_state, p.dy, p.d_final_state = ptr(S0), ptr(dY), ptr(dSf)
     p.dx, p.ddt, p.dA, p.dB, p.dC, p.dD, p.d_initial_state = ptr(dX), ptr(ddt), ptr(dA), ptr(dB), ptr(dC), ptr(dD), ptr(dS0)
-    p.y_stride_b, p.y_stride_l, p.y_stride_h = _strides3(Y)
     p.dy_stride_b, p.dy_stride_l, p.dy_stride_h = _strides3(dY)
     p.dx_stride_b, p.dx_stride_l, p.dx_stride_h = _strides3(dX)
     p.ddt_stride_b, p.ddt_stride_l = ddt.stride(0), ddt.stride(1)
@@ -133,9 +132,8 @@ class Mamba2Kernel(torch.autograd.Function):
     @staticmethod
     def forward(ctx, dt, A, X, B, C, D, initial_state=None, return_final_state=False):
         Y, S = ssd_forward(dt, A, X, B, C, D, initial_state, return_final_state)
-        # inputs are saved as in the reference (:492); the output is saved as well because the
-        # decay gradient is formed from dy . y instead of being re-derived from C o dC - B o dB
-        ctx.save_for_backward(dt, A, X, B, C, D, initial_state, Y)
+        # only the inputs are saved, as in the reference (:492); the backward recomputes per chunk
+        ctx.save_for_backward(dt, A, X, B, C, D, initial_state)
         ctx.return_final_state = return_final_state
         if return_final_state:
             return Y, S
@@ -143,10 +141,10 @@ class Mamba2Kernel(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, d_output, *rest):
-        dt, A, X, B, C, D, initial_state, Y = ctx.saved_tensors
+        dt, A, X, B, C, D, initial_state = ctx.saved_tensors
         dS = rest[0] if (ctx.return_final_state and rest and rest[0] is not None) else None
         want_dinit = initial_state is not None and ctx.needs_input_grad[6]
-        ddt, dA, dX, dB, dC, dD, dS0 = ssd_backward(dt, A, X, B, C, D, Y, d_output, initial_state, dS, want_dinit)
+        ddt, dA, dX, dB, dC, dD, dS0 = ssd_backward(dt, A, X, B, C, D, d_output, initial_state, dS, want_dinit)
         dA = dA.to(A.dtype)
         dD = dD.to(D.dtype) if D is not None else None
         return ddt, dA, dX, dB, dC, dD, dS0, None

@@ -59,8 +59,13 @@ def test_ssd_forward_initial_state_no_D_fp32_dt(dtype):
     y_ref, S_ref = ssd_chunked_ref(r["dt"], r["A"], r["X"], r["B"], r["C"], None, initial_state=S0.double(), chunk=128)
     dd = _dev(d)
     y, S = mamba2_kernel(dd["dt"], dd["A"], dd["X"], dd["B"], dd["C"], None, initial_state=S0.to(DEV), return_final_state=True)
-    tol, metric = _tol(dtype)
-    assert metric(y, y_ref) < tol and metric(S, S_ref) < tol
+    if dtype == torch.float32:
+        assert rel_err(y, y_ref) < 1e-4 and rel_err(S, S_ref) < 1e-4
+    else:
+        # Without the D x skip the outputs are heavy-tailed (max |y| ~ 25 RMS here), and rounding the MFMA
+        # operands to bf16 (2^-9 relative each: decay*G tile, carried state) gives errors proportional to
+        # the largest outputs; the bound is therefore taken against max |y|: 1e-2.
+        assert rel_err(y, y_ref) < 1e-2 and rel_rms_err(S, S_ref) < 2e-2
 
 
 def test_ssd_packed_views():
