@@ -1,0 +1,205 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X Mamba-2 mixer hot path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|ssd|conv|decode] [--no-cpu]
+
+One "step" is one pass of the hot path over one batch of synthetic input, inputs resident in HBM:
+  ssd    : SSD chunked scan fwd+bwd, bf16, 2.7B shape (b4, l2048, h80, p64, n128, g1, chunk 128)   <- headline
+  conv   : depthwise conv1d k=4 + SiLU fwd+bwd, bf16 (b4, l2048, C5376)
+  decode : one decode token-step over 64 stacked layers of the 2.7B shape, batch 128
+Prints ONE JSON line (rank 0).  The headline metric is SSD fwd+bwd tokens/s; `roofline` prices the
+SSD step against the dense bf16 MFMA peak using the ALGORITHMIC FLOPs (G shared per group, no
+recompute counted); conv and decode are reported under `other` against the HBM peak with their
+algorithmic bytes.  `cpu_baseline` is the pure-PyTorch oracle timed on this box's host cores.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "state-space-models-neuron_amd"))
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0     # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0              # MI355X HBM3E
+
+SSD_CFG = dict(b=4, l=2048, h=80, p=64, n=128, g=1)
+CONV_CFG = dict(b=4, l=2048, C=5376, k=4)
+DEC_CFG = dict(b=128, h=80, p=64, n=128, g=1, k=4, W=3, layers=64)
+Q = 128
+
+
+def ssd_flops_fwd(b, l, h, p, n, g):
+    c = math.ceil(l / Q)
+    return b * c * (h * (2 * Q * Q * p + 4 * Q * n * p) + g * 2 * Q * Q * n)
+
+
+def event_time_ms(fn, steps, warmup):
+    """Per-step durations from HIP events recorded on the stream the kernels are launched on."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for s, e in evs:
+        s.record()
+        fn()
+        e.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    per = [s.elapsed_time(e) for s, e in evs]
+    return wall, per
+
+
+def bench_ssd(steps, warmup):
+    import torch
+    from mamba2.mamba2_kernel import ssd_backward, ssd_forward
+    from oracle.ssd import make_ssd_inputs
+    cfg = SSD_CFG
+    d = make_ssd_inputs(cfg["b"], cfg["l"], cfg["h"], cfg["p"], cfg["n"], cfg["g"], seed=0, dtype=torch.bfloat16, device="cuda:0")
+
+    def step():
+        y, _ = ssd_forward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"])
+        ssd_backward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], d["dy"])
+
+    wall_ms, per = event_time_ms(step, steps, warmup)
+    per.sort()
+    ms = sum(per) / len(per)
+    tokens = cfg["b"] * cfg["l"]
+    flops = 3 * ssd_flops_fwd(**cfg)
+    return dict(ms_per_step=wall_ms, ms_event_avg=ms, ms_event_min=per[0], ms_event_median=per[len(per) // 2],
+                tokens_per_s=tokens / (wall_ms * 1e-3), flops=flops, tflops=flops / (ms * 1e-3) / 1e12, tokens=tokens)
+
+
+def bench_conv(steps, warmup):
+    import torch
+    from mamba2.conv1d_grouped import conv1d_backward, conv1d_forward
+    from oracle.conv import make_conv_inputs
+    cfg = CONV_CFG
+    nsets = 4          # rotate input sets so the 256 MB MALL does not serve the reads
+    sets = [make_conv_inputs(cfg["b"], cfg["l"], cfg["C"], cfg["k"], seed=s, dtype=torch.bfloat16, device="cuda:0") for s in range(nsets)]
+    outs = [torch.empty_like(sets[0]["x"]) for _ in range(2)]
+    state = {"i": 0}
+
+    def step():
+        d = sets[state["i"] % nsets]
+        state["i"] += 1
+        conv1d_forward(d["x"], d["w"], d["bias"], "silu", channels_last=True, out=outs[0])
+        conv1d_backward(d["x"], d["w"], d["bias"], d["dy"], "silu", channels_last=True, out_dx=outs[1])
+
+    wall_ms, per = event_time_ms(step, steps, warmup)
+    ms = sum(per) / len(per)
+    elems = cfg["b"] * cfg["l"] * cfg["C"]
+    bytes_ = elems * 2 * 5          # fwd: read x, write y; bwd: read x, dy, write dx
+    tokens = cfg["b"] * cfg["l"]
+    return dict(metric="conv1d+SiLU fwd+bwd tokens/s", value=tokens / (ms * 1e-3), unit="tokens/s", ms_per_step=ms, dtype="bf16",
+                config={"workload": "depthwise conv1d k=4 + SiLU fwd+bwd, b4 l2048 C5376, channels-last"},
+                roofline={"bound": "hbm", "achieved": bytes_ / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                          "algorithmic_bytes_per_step": bytes_, "kernels": "conv_fwd_cl_kernel + conv_bwd_cl_kernel + conv_reduce_partials_kernel"})
+
+
+def bench_decode(steps, warmup):
+    import torch
+    from mamba2.mamba2_kernel_inference import mamba2_kernel_inference
+    from oracle.decode import make_decode_inputs
+    cfg = DEC_CFG
+    L = cfg["layers"]
+    d = make_decode_inputs(cfg["b"], cfg["h"], cfg["p"], cfg["n"], cfg["g"], cfg["k"], cfg["W"], seed=0, act_dtype=torch.bfloat16, device="cuda:0")
+    gen = torch.Generator(device="cuda:0").manual_seed(1)
+    # distinct state buffers per layer (21.5 GB of fp32 SSM state): nothing is served from cache
+    S = [0.1 * torch.randn(cfg["b"], cfg["h"], cfg["p"], cfg["n"], device="cuda:0", generator=gen) for _ in range(L)]
+    conv = [torch.randn(cfg["b"], d["xBC"].shape[-1], cfg["W"], device="cuda:0", generator=gen).to(torch.bfloat16) for _ in range(L)]
+
+    def step():
+        for i in range(L):
+            mamba2_kernel_inference(d["xBC"], conv[i], d["conv_weight"], d["conv_bias"], S[i], d["dt"], d["A"], d["D"], n_groups=cfg["g"])
+
+    wall_ms, per = event_time_ms(step, steps, warmup)
+    ms = sum(per) / len(per)
+    Cx = d["xBC"].shape[-1]
+    per_layer = 2 * S[0].numel() * 4 + 2 * conv[0].numel() * 2 + cfg["b"] * Cx * 2 + cfg["b"] * cfg["h"] * 2 + cfg["b"] * cfg["h"] * cfg["p"] * 2
+    bytes_ = per_layer * L
+    return dict(metric="decode token-step latency (64 layers, batch 128)", value=ms * 1e3, unit="us/step", higher_is_better=False,
+                us_per_sequence_token=ms * 1e3 / cfg["b"], ms_per_step=ms, wall_ms_per_step=wall_ms, dtype="f32 state / bf16 activations",
+                config={"workload": "decode step, 64 layers x (b128, h80, p64, n128, C5376, W3), states in place"},
+                roofline={"bound": "hbm", "achieved": bytes_ / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                          "algorithmic_bytes_per_step": bytes_, "kernels": "decode_conv_kernel + decode_ssm_kernel, 64 launches each"})
+
+
+def cpu_baseline_ssd():
+    """The pure-PyTorch chunked oracle (fp32, autograd) on the host cores: the full headline configuration."""
+    import torch
+    from oracle.ssd import make_ssd_inputs, ssd_grads_ref
+    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+    torch.set_num_threads(cores)
+    cfg = SSD_CFG
+    d = make_ssd_inputs(cfg["b"], cfg["l"], cfg["h"], cfg["p"], cfg["n"], cfg["g"], seed=0, dtype=torch.float32)
+    times = []
+    for i in range(3):
+        t0 = time.perf_counter()
+        ssd_grads_ref(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], d["dy"], chunk=Q)
+        times.append(time.perf_counter() - t0)
+    t = sorted(times[1:])[0] if len(times) > 1 else times[0]
+    return {"value": cfg["b"] * cfg["l"] / t, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "full workload (b4 l2048 h80 p64 n128), fp32, chunked-matmul oracle with autograd, 1 warm-up + best of 2",
+            "seconds_per_step": t}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="all", choices=["all", "ssd", "conv", "decode"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the hot path has no collective); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from mamba2 import _lib
+    _lib.load()          # fails loudly when the HIP library is missing
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+
+    out = {}
+    other = {}
+    if a.workload in ("all", "ssd"):
+        r = bench_ssd(a.steps, a.warmup)
+        out.update({
+            "metric": "SSD fwd+bwd tokens/s", "value": r["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1,
+            "steps": a.steps, "warmup": a.warmup, "ms_per_step": r["ms_per_step"], "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "Mamba-2 2.7B-shaped SSD chunked scan fwd+bwd: b4 l2048 h80 p64 n128 g1 chunk128, bf16 I/O, fp32 state"},
+            "roofline": {"bound": "mfma", "achieved": r["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": r["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                         "algorithmic_flops_per_step": r["flops"], "event_ms_avg": r["ms_event_avg"],
+                         "event_ms_min": r["ms_event_min"],
+                         "kernels": "all launches of m2_ssd_fwd + m2_ssd_bwd (one step), HIP events on the launch stream"},
+        })
+    if a.workload in ("all", "conv"):
+        other["conv1d"] = bench_conv(a.steps, a.warmup)
+    if a.workload in ("all", "decode"):
+        other["decode"] = bench_decode(max(3, a.steps // 4), max(1, a.warmup // 2))
+    if a.workload not in ("all", "ssd"):
+        key = "conv1d" if a.workload == "conv" else "decode"
+        out.update(other.pop(key))
+        out.update({"n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "scaling": "weak", "vs_baseline": None, "data": "synthetic"})
+        out.setdefault("higher_is_better", True)
+    if other:
+        out["other"] = other
+    if not a.no_cpu and a.workload in ("all", "ssd"):
+        out["cpu_baseline"] = cpu_baseline_ssd()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

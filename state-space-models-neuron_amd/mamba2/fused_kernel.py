@@ -1,0 +1,131 @@
+"""Mixer core ``zxBCdt -> norm_out`` with the reference's signatures (``mamba2/fused_kernel.py:423-487``):
+
+    mamba2_fused_kernel(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias, norm_weight,
+                        n_groups, ssm_state_size, intermediate_size, head_dim) -> norm_out[b,l,d_inner]
+
+Pipeline (``fused_kernel.py:252-282``): split [z | xBC | dt] -> depthwise conv + SiLU ->
+softplus(dt + dt_bias) -> SSD scan -> gated RMSNorm per group (eps 1e-5).
+
+The split is never materialised: the HIP kernels take strided views of ``zxBCdt`` (the conv reads
+the xBC columns in place; the scan reads x, B, C as views of the conv output), and in the backward
+the scan writes dx, dB, dC straight into one packed buffer and the conv writes its dx straight into
+the xBC columns of ``d_zxBCdt``.  ``Mamba2FusedKernel`` saves only its inputs and recomputes conv,
+softplus and scan in the backward (as the reference does, ``:352-367``); ``...WithCaching`` keeps the
+intermediates (``:449-471``).
+"""
+import torch
+
+from . import glue
+from .conv1d_grouped import conv1d_backward, conv1d_forward
+from .mamba2_kernel import ssd_backward, ssd_forward
+
+NORM_EPS = 1e-5     # fixed in the reference's fused kernel (fused_kernel.py:254)
+
+
+def _views(zxBCdt, n_groups, d_state, d_inner, d_head):
+    b, l, width = zxBCdt.shape
+    h = d_inner // d_head
+    d_conv = d_inner + 2 * n_groups * d_state
+    if width != d_inner + d_conv + h:
+        raise ValueError(f"zxBCdt width {width} != 2*d_inner + 2*g*n + h = {d_inner + d_conv + h}")
+    z = zxBCdt[..., :d_inner]
+    xBC = zxBCdt[..., d_inner:d_inner + d_conv]
+    dt = zxBCdt[..., d_inner + d_conv:]
+    return z, xBC, dt, h, d_conv
+
+
+def _xbc_views(conv_out, n_groups, d_state, d_inner, d_head):
+    h = d_inner // d_head
+    gn = n_groups * d_state
+    x = conv_out[..., :d_inner].unflatten(-1, (h, d_head))
+    Bm = conv_out[..., d_inner:d_inner + gn].unflatten(-1, (n_groups, d_state))
+    Cm = conv_out[..., d_inner + gn:].unflatten(-1, (n_groups, d_state))
+    return x, Bm, Cm
+
+
+def _forward_parts(zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, n_groups, d_state, d_inner, d_head):
+    z, xBC, dt, h, d_conv = _views(zxBCdt, n_groups, d_state, d_inner, d_head)
+    b, l, _ = zxBCdt.shape
+    conv_out = torch.empty((b, l, d_conv), dtype=zxBCdt.dtype, device=zxBCdt.device)
+    conv1d_forward(xBC, conv_w, conv_b, "silu", channels_last=True, out=conv_out)
+    dt_sp = glue.softplus_bias(dt, dt_bias)
+    x, Bm, Cm = _xbc_views(conv_out, n_groups, d_state, d_inner, d_head)
+    y, _ = ssd_forward(dt_sp, logA, x, Bm, Cm, D)
+    scan_out = y.view(b, l, d_inner)
+    norm_out = glue.rmsnorm_gated(scan_out, z, norm_w, n_groups, NORM_EPS, out_dtype=zxBCdt.dtype)
+    return norm_out, conv_out, dt_sp, scan_out
+
+
+def _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out,
+                    n_groups, d_state, d_inner, d_head):
+    z, xBC, dt, h, d_conv = _views(zxBCdt, n_groups, d_state, d_inner, d_head)
+    b, l, width = zxBCdt.shape
+    d_zxBCdt = torch.empty_like(zxBCdt, memory_format=torch.contiguous_format)
+    dz_view = d_zxBCdt[..., :d_inner]
+    dxBC_view = d_zxBCdt[..., d_inner:d_inner + d_conv]
+    ddt_view = d_zxBCdt[..., d_inner + d_conv:]
+    # gated RMSNorm backward: d_scan_out, d_z (written into d_zxBCdt), d_norm_weight
+    d_scan_out, d_norm_w = glue.rmsnorm_gated_bwd(scan_out, z, norm_w, d_output, n_groups, NORM_EPS, out_dz=dz_view)
+    # SSD backward, gradients of x, B, C written into one packed [dx | dB | dC] buffer
+    x, Bm, Cm = _xbc_views(conv_out, n_groups, d_state, d_inner, d_head)
+    d_conv_out = torch.empty_like(conv_out)
+    dx_v, dB_v, dC_v = _xbc_views(d_conv_out, n_groups, d_state, d_inner, d_head)
+    d_dt_sp, d_logA, _, _, _, d_D, _ = ssd_backward(dt_sp, logA, x, Bm, Cm, D, d_scan_out.view(b, l, h, d_head),
+                                                     out_dX=dx_v, out_dB=dB_v, out_dC=dC_v)
+    # softplus backward (into the dt columns) and conv backward (into the xBC columns)
+    d_dt_bias = glue.softplus_bias_bwd(dt, dt_bias, d_dt_sp, out_d_in=ddt_view)
+    _, d_conv_w, d_conv_b = conv1d_backward(xBC, conv_w, conv_b, d_conv_out, "silu", channels_last=True, out_dx=dxBC_view)
+    return (d_zxBCdt, d_logA.to(logA.dtype), d_D.to(D.dtype) if D is not None else None, d_conv_w, d_conv_b,
+            d_dt_bias.to(dt_bias.dtype), d_norm_w.to(norm_w.dtype))
+
+
+class Mamba2FusedKernel(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias,
+                norm_weight, n_groups, ssm_state_size, intermediate_size, head_dim):
+        norm_out, *_ = _forward_parts(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias, norm_weight,
+                                      n_groups, ssm_state_size, intermediate_size, head_dim)
+        ctx.dims = (n_groups, ssm_state_size, intermediate_size, head_dim)
+        ctx.save_for_backward(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias, norm_weight)
+        return norm_out
+
+    @staticmethod
+    def backward(ctx, d_output):
+        zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w = ctx.saved_tensors
+        # recompute conv, softplus and scan (only the inputs were saved)
+        _, conv_out, dt_sp, scan_out = _forward_parts(zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, *ctx.dims)
+        grads = _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out, *ctx.dims)
+        return (*grads, None, None, None, None)
+
+
+class Mamba2FusedKernelWithCaching(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias,
+                norm_weight, n_groups, ssm_state_size, intermediate_size, head_dim):
+        norm_out, conv_out, dt_sp, scan_out = _forward_parts(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias, norm_weight,
+                                                             n_groups, ssm_state_size, intermediate_size, head_dim)
+        ctx.dims = (n_groups, ssm_state_size, intermediate_size, head_dim)
+        ctx.save_for_backward(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias, norm_weight, conv_out, dt_sp, scan_out)
+        return norm_out
+
+    @staticmethod
+    def backward(ctx, d_output):
+        zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out = ctx.saved_tensors
+        grads = _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out, *ctx.dims)
+        return (*grads, None, None, None, None)
+
+
+def mamba2_fused_kernel(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias,
+                        norm_weight, n_groups, ssm_state_size, intermediate_size,
+                        head_dim):
+    return Mamba2FusedKernel.apply(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias,
+                                   norm_weight, n_groups, ssm_state_size, intermediate_size,
+                                   head_dim)
+
+
+def mamba2_fused_kernel_with_caching(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias,
+                                     norm_weight, n_groups, ssm_state_size, intermediate_size,
+                                     head_dim):
+    return Mamba2FusedKernelWithCaching.apply(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias,
+                                              norm_weight, n_groups, ssm_state_size, intermediate_size,
+                                              head_dim)
