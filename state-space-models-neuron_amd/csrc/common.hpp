@@ -59,6 +59,42 @@ __device__ __forceinline__ void store16(T* __restrict__ p, const float (&in)[Vec
     *reinterpret_cast<uint4*>(p) = raw;
 }
 
+// Raw vector of V elements of T (8 or 16 bytes), kept unconverted in registers until used.
+template <int BYTES> struct RawBytes;
+template <> struct RawBytes<16> { using type = uint4; };
+template <> struct RawBytes<8> { using type = uint2; };
+template <> struct RawBytes<4> { using type = uint32_t; };
+template <typename T, int V> using RawVec = typename RawBytes<V * (int)sizeof(T)>::type;
+template <typename T, int V>
+__device__ __forceinline__ RawVec<T, V> loadv_raw(const T* __restrict__ p) { return *reinterpret_cast<const RawVec<T, V>*>(p); }
+template <typename T, int V>
+__device__ __forceinline__ void cvtv(const RawVec<T, V>& raw, float (&out)[V]) {
+    const T* e = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+    for (int i = 0; i < V; ++i) out[i] = to_f32(e[i]);
+}
+template <typename T, int V>
+__device__ __forceinline__ void loadv(const T* __restrict__ p, float (&out)[V]) { cvtv<T, V>(loadv_raw<T, V>(p), out); }
+template <typename T, int V>
+__device__ __forceinline__ void storev(T* __restrict__ p, const float (&in)[V]) {
+    RawVec<T, V> raw;
+    T* e = reinterpret_cast<T*>(&raw);
+#pragma unroll
+    for (int i = 0; i < V; ++i) e[i] = from_f32<T>(in[i]);
+    *reinterpret_cast<RawVec<T, V>*>(p) = raw;
+}
+
+// raw 16-byte load (kept unconverted in 4 registers until used) and its conversion
+template <typename T>
+__device__ __forceinline__ uint4 load16_raw(const T* __restrict__ p) { return *reinterpret_cast<const uint4*>(p); }
+template <typename T>
+__device__ __forceinline__ void cvt16(const uint4& raw, float (&out)[VecTraits<T>::kVec]) {
+    constexpr int N = VecTraits<T>::kVec;
+    const T* e = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+    for (int i = 0; i < N; ++i) out[i] = to_f32(e[i]);
+}
+
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + __expf(-z)); }
 // d/dz silu(z) = s * (1 + z * (1 - s)),  s = sigmoid(z)
 __device__ __forceinline__ float silu_grad_f(float z) {

@@ -23,7 +23,20 @@ namespace m2 {
 namespace {
 
 constexpr int kMaxK = 8;
-constexpr int kTL = 32;        // tokens per thread in the fast path
+#ifndef M2_CONV_TL
+#define M2_CONV_TL 64
+#endif
+#ifndef M2_CONV_UNR
+#define M2_CONV_UNR 4
+#endif
+#ifndef M2_CONV_VF
+#define M2_CONV_VF 8
+#endif
+#ifndef M2_CONV_VB
+#define M2_CONV_VB 8
+#endif
+constexpr int kTL = M2_CONV_TL;      // tokens per thread in the fast path
+constexpr int kUNR = M2_CONV_UNR;    // tokens whose loads are in flight together
 constexpr int kCVT = 32;       // channel vectors per block (x dimension)
 constexpr int kSEG = 8;        // token segments per block (y dimension)
 
@@ -38,12 +51,11 @@ __device__ __forceinline__ void st_param(void* p, int pd, int64_t i, float v) {
 // ------------------------------------------------------------------------------------------
 // Fast path, channels-last, k == 4.
 // grid: x = ceil(CV / kCVT), y = ceil(nseg / kSEG), z = batch; block (kCVT, kSEG).
-template <typename T, int ACT>
+template <typename T, int V, int ACT>
 __global__ void __launch_bounds__(kCVT * kSEG)
 conv_fwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const void* __restrict__ bias,
                    T* __restrict__ y, int64_t l, int64_t C, int64_t xsb, int64_t xsl, int64_t ysb, int64_t ysl,
                    int pd) {
-    constexpr int V = VecTraits<T>::kVec;
     const int64_t cv = (int64_t)blockIdx.x * kCVT + threadIdx.x;
     const int64_t seg = (int64_t)blockIdx.y * kSEG + threadIdx.y;
     const int64_t b = blockIdx.z;
@@ -63,34 +75,48 @@ conv_fwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const vo
     float h0[V], h1[V], h2[V];   // x[t-3], x[t-2], x[t-1]
 #pragma unroll
     for (int j = 0; j < V; ++j) h0[j] = h1[j] = h2[j] = 0.f;
-    if (t0 - 3 >= 0) load16(xp + (t0 - 3) * xsl, h0);
-    if (t0 - 2 >= 0) load16(xp + (t0 - 2) * xsl, h1);
-    if (t0 - 1 >= 0) load16(xp + (t0 - 1) * xsl, h2);
+    if (t0 - 3 >= 0) loadv<T, V>(xp + (t0 - 3) * xsl, h0);
+    if (t0 - 2 >= 0) loadv<T, V>(xp + (t0 - 2) * xsl, h1);
+    if (t0 - 1 >= 0) loadv<T, V>(xp + (t0 - 1) * xsl, h2);
     const int64_t t1 = (t0 + kTL < l) ? t0 + kTL : l;
-#pragma unroll 4
-    for (int64_t t = t0; t < t1; ++t) {
-        float cur[V], out[V];
-        load16(xp + t * xsl, cur);
+    // software pipeline: the loads of group g+1 are issued before group g is computed and stored
+    RawVec<T, V> nxt[kUNR];
 #pragma unroll
-        for (int j = 0; j < V; ++j) {
-            float z = bv[j] + wv[0][j] * h0[j] + wv[1][j] * h1[j] + wv[2][j] * h2[j] + wv[3][j] * cur[j];
-            out[j] = act_f<ACT>(z);
-            h0[j] = h1[j]; h1[j] = h2[j]; h2[j] = cur[j];
+    for (int u = 0; u < kUNR; ++u)
+        if (t0 + u < t1) nxt[u] = loadv_raw<T, V>(xp + (t0 + u) * xsl);
+    for (int64_t tg = t0; tg < t1; tg += kUNR) {
+        RawVec<T, V> raw[kUNR];
+#pragma unroll
+        for (int u = 0; u < kUNR; ++u) raw[u] = nxt[u];
+#pragma unroll
+        for (int u = 0; u < kUNR; ++u)
+            if (tg + kUNR + u < t1) nxt[u] = loadv_raw<T, V>(xp + (tg + kUNR + u) * xsl);
+#pragma unroll
+        for (int u = 0; u < kUNR; ++u) {
+            if (tg + u < t1) {
+                float out[V], cur[V];
+                cvtv<T, V>(raw[u], cur);
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    float z = bv[j] + wv[0][j] * h0[j] + wv[1][j] * h1[j] + wv[2][j] * h2[j] + wv[3][j] * cur[j];
+                    out[j] = act_f<ACT>(z);
+                    h0[j] = h1[j]; h1[j] = h2[j]; h2[j] = cur[j];
+                }
+                storev<T, V>(yp + (tg + u) * ysl, out);
+            }
         }
-        store16(yp + t * ysl, out);
     }
 }
 
 // Backward fast path.  Each thread marches t over [t0, t0+TL+3): at step t it forms g[t] and
 // emits dx[t-3] = w3 g[t-3] + w2 g[t-2] + w1 g[t-1] + w0 g[t]  (dx[s] = sum_i w[i] g[s+3-i]).
 // Partials: part[(blockIdx.z * gridDim.y + blockIdx.y)][c][0..4] = (dw0..dw3, db).
-template <typename T, int ACT>
+template <typename T, int V, int ACT>
 __global__ void __launch_bounds__(kCVT * kSEG)
 conv_bwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const void* __restrict__ bias,
                    const T* __restrict__ dy, T* __restrict__ dx, float* __restrict__ part,
                    int64_t l, int64_t C, int64_t xsb, int64_t xsl, int64_t gsb, int64_t gsl,
                    int64_t dsb, int64_t dsl, int pd) {
-    constexpr int V = VecTraits<T>::kVec;
     __shared__ float red[kSEG][5][kCVT * V + 1];
     const int64_t cv = (int64_t)blockIdx.x * kCVT + threadIdx.x;
     const int64_t seg = (int64_t)blockIdx.y * kSEG + threadIdx.y;
@@ -120,43 +146,62 @@ conv_bwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const vo
         float g0[V], g1[V], g2[V];   // g[t-3..t-1]
 #pragma unroll
         for (int j = 0; j < V; ++j) h0[j] = h1[j] = h2[j] = g0[j] = g1[j] = g2[j] = 0.f;
-        if (t0 - 3 >= 0) load16(xp + (t0 - 3) * xsl, h0);
-        if (t0 - 2 >= 0) load16(xp + (t0 - 2) * xsl, h1);
-        if (t0 - 1 >= 0) load16(xp + (t0 - 1) * xsl, h2);
+        if (t0 - 3 >= 0) loadv<T, V>(xp + (t0 - 3) * xsl, h0);
+        if (t0 - 2 >= 0) loadv<T, V>(xp + (t0 - 2) * xsl, h1);
+        if (t0 - 1 >= 0) loadv<T, V>(xp + (t0 - 1) * xsl, h2);
         const int64_t tseg = (t0 + kTL < l) ? t0 + kTL : l;      // end of this thread's own tokens
         const int64_t tend = tseg + 3;                            // march 3 further for the dx lag
-#pragma unroll 2
-        for (int64_t t = t0; t < tend; ++t) {
-            float cur[V], gy[V], g[V];
-            if (t < l) { load16(xp + t * xsl, cur); load16(gp + t * gsl, gy); }
-            else {
+        // software pipeline: the loads of group g+1 are issued before group g is computed and stored
+        RawVec<T, V> nx[kUNR], ng[kUNR];
 #pragma unroll
-                for (int j = 0; j < V; ++j) cur[j] = gy[j] = 0.f;
+        for (int u = 0; u < kUNR; ++u) {
+            const int64_t t = t0 + u;
+            if (t < tend && t < l) { nx[u] = loadv_raw<T, V>(xp + t * xsl); ng[u] = loadv_raw<T, V>(gp + t * gsl); }
+            else { nx[u] = RawVec<T, V>{}; ng[u] = RawVec<T, V>{}; }
+        }
+        for (int64_t tg = t0; tg < tend; tg += kUNR) {
+            RawVec<T, V> rawx[kUNR], rawg[kUNR];
+#pragma unroll
+            for (int u = 0; u < kUNR; ++u) { rawx[u] = nx[u]; rawg[u] = ng[u]; }
+#pragma unroll
+            for (int u = 0; u < kUNR; ++u) {
+                const int64_t t = tg + kUNR + u;
+                if (t < tend && t < l) { nx[u] = loadv_raw<T, V>(xp + t * xsl); ng[u] = loadv_raw<T, V>(gp + t * gsl); }
+                else { nx[u] = RawVec<T, V>{}; ng[u] = RawVec<T, V>{}; }
             }
-            const bool own = t < tseg;
 #pragma unroll
-            for (int j = 0; j < V; ++j) {
-                float z = bv[j] + wv[0][j] * h0[j] + wv[1][j] * h1[j] + wv[2][j] * h2[j] + wv[3][j] * cur[j];
-                g[j] = gy[j] * act_grad_f<ACT>(z);     // gy == 0 beyond the sequence end
-                if (own) {
-                    acc[0][j] += h0[j] * g[j];
-                    acc[1][j] += h1[j] * g[j];
-                    acc[2][j] += h2[j] * g[j];
-                    acc[3][j] += cur[j] * g[j];
-                    acc[4][j] += g[j];
+            for (int u = 0; u < kUNR; ++u) {
+                const int64_t t = tg + u;
+                if (t < tend) {
+                    const bool own = t < tseg;
+                    float g[V], cur[V], gy[V];
+                    cvtv<T, V>(rawx[u], cur);
+                    cvtv<T, V>(rawg[u], gy);
+#pragma unroll
+                    for (int j = 0; j < V; ++j) {
+                        float z = bv[j] + wv[0][j] * h0[j] + wv[1][j] * h1[j] + wv[2][j] * h2[j] + wv[3][j] * cur[j];
+                        g[j] = gy[j] * act_grad_f<ACT>(z);     // gy == 0 beyond the sequence end
+                        if (own) {
+                            acc[0][j] += h0[j] * g[j];
+                            acc[1][j] += h1[j] * g[j];
+                            acc[2][j] += h2[j] * g[j];
+                            acc[3][j] += cur[j] * g[j];
+                            acc[4][j] += g[j];
+                        }
+                    }
+                    if (t - 3 >= t0) {
+                        float o[V];
+#pragma unroll
+                        for (int j = 0; j < V; ++j)
+                            o[j] = wv[3][j] * g0[j] + wv[2][j] * g1[j] + wv[1][j] * g2[j] + wv[0][j] * g[j];
+                        storev<T, V>(dp + (t - 3) * dsl, o);
+                    }
+#pragma unroll
+                    for (int j = 0; j < V; ++j) {
+                        h0[j] = h1[j]; h1[j] = h2[j]; h2[j] = cur[j];
+                        g0[j] = g1[j]; g1[j] = g2[j]; g2[j] = g[j];
+                    }
                 }
-            }
-            if (t - 3 >= t0) {
-                float o[V];
-#pragma unroll
-                for (int j = 0; j < V; ++j)
-                    o[j] = wv[3][j] * g0[j] + wv[2][j] * g1[j] + wv[1][j] * g2[j] + wv[0][j] * g[j];
-                store16(dp + (t - 3) * dsl, o);
-            }
-#pragma unroll
-            for (int j = 0; j < V; ++j) {
-                h0[j] = h1[j]; h1[j] = h2[j]; h2[j] = cur[j];
-                g0[j] = g1[j]; g1[j] = g2[j]; g2[j] = g[j];
             }
         }
     }
@@ -286,17 +331,21 @@ conv_bwd_dw_generic_kernel(const T* __restrict__ x, const void* __restrict__ w, 
     }
 }
 
-template <typename T>
+// elements per thread: 16-byte vectors forward, 8-byte vectors backward (the backward carries twice the
+// per-channel state in registers; halving the vector keeps its occupancy up)
+template <typename T> constexpr int conv_vec(bool bwd) { return (int)(bwd ? M2_CONV_VB / sizeof(T) : M2_CONV_VF / sizeof(T)); }
+
+template <typename T, int V>
 bool fast_path_ok(const m2_conv1d_params* p, bool bwd) {
-    constexpr int V = VecTraits<T>::kVec;
     if (p->k != 4 || p->x_stride_c != 1 || p->y_stride_c != 1) return false;
     if (p->channels % V) return false;
     if (p->x_stride_b % V || p->x_stride_l % V || p->y_stride_b % V || p->y_stride_l % V) return false;
-    if (!aligned16(p->x)) return false;
-    if (!bwd && !aligned16(p->y)) return false;
+    auto al = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) % (V * sizeof(T))) == 0; };
+    if (!al(p->x)) return false;
+    if (!bwd && !al(p->y)) return false;
     if (bwd) {
         if (p->dx_stride_c != 1 || p->dx_stride_b % V || p->dx_stride_l % V) return false;
-        if (!aligned16(p->dy) || !aligned16(p->dx)) return false;
+        if (!al(p->dy) || !al(p->dx)) return false;
     }
     return true;
 }
@@ -317,16 +366,16 @@ int launch_fwd(const m2_conv1d_params* p, hipStream_t st) {
     const int64_t nb = p->batch, l = p->seqlen, C = p->channels;
     const T* x = static_cast<const T*>(p->x);
     T* y = static_cast<T*>(p->y);
-    if (fast_path_ok<T>(p, false) && p->activation != M2_ACT_RELU) {
-        constexpr int V = VecTraits<T>::kVec;
+    constexpr int V = conv_vec<T>(false);
+    if (fast_path_ok<T, V>(p, false) && p->activation != M2_ACT_RELU) {
         const int64_t CV = C / V, nseg = ceil_div(l, kTL);
         dim3 grid((unsigned)ceil_div(CV, kCVT), (unsigned)ceil_div(nseg, kSEG), (unsigned)nb), block(kCVT, kSEG);
         M2_REQUIRE(grid.y <= 65535, M2_ERR_SHAPE, "conv1d: sequence too long for the grid");
         if (p->activation == M2_ACT_SILU)
-            conv_fwd_cl_kernel<T, M2_ACT_SILU><<<grid, block, 0, st>>>(x, p->w, p->bias, y, l, C, p->x_stride_b, p->x_stride_l,
+            conv_fwd_cl_kernel<T, V, M2_ACT_SILU><<<grid, block, 0, st>>>(x, p->w, p->bias, y, l, C, p->x_stride_b, p->x_stride_l,
                                                                         p->y_stride_b, p->y_stride_l, p->param_dtype);
         else
-            conv_fwd_cl_kernel<T, M2_ACT_NONE><<<grid, block, 0, st>>>(x, p->w, p->bias, y, l, C, p->x_stride_b, p->x_stride_l,
+            conv_fwd_cl_kernel<T, V, M2_ACT_NONE><<<grid, block, 0, st>>>(x, p->w, p->bias, y, l, C, p->x_stride_b, p->x_stride_l,
                                                                         p->y_stride_b, p->y_stride_l, p->param_dtype);
     } else {
         const int64_t total = nb * l * C;
@@ -344,8 +393,8 @@ int launch_bwd(const m2_conv1d_params* p, hipStream_t st) {
     const T* x = static_cast<const T*>(p->x);
     const T* dy = static_cast<const T*>(p->dy);
     T* dx = static_cast<T*>(p->dx);
-    if (fast_path_ok<T>(p, true) && p->activation != M2_ACT_RELU) {
-        constexpr int V = VecTraits<T>::kVec;
+    constexpr int V = conv_vec<T>(true);
+    if (fast_path_ok<T, V>(p, true) && p->activation != M2_ACT_RELU) {
         const int64_t CV = C / V, nseg = ceil_div(l, kTL);
         dim3 grid((unsigned)ceil_div(CV, kCVT), (unsigned)ceil_div(nseg, kSEG), (unsigned)nb), block(kCVT, kSEG);
         M2_REQUIRE(grid.y <= 65535, M2_ERR_SHAPE, "conv1d: sequence too long for the grid");
@@ -355,10 +404,10 @@ int launch_bwd(const m2_conv1d_params* p, hipStream_t st) {
                    "conv1d_bwd: workspace %zu bytes < %zu needed", p->workspace_bytes, need);
         float* part = static_cast<float*>(p->workspace);
         if (p->activation == M2_ACT_SILU)
-            conv_bwd_cl_kernel<T, M2_ACT_SILU><<<grid, block, 0, st>>>(x, p->w, p->bias, dy, dx, part, l, C, p->x_stride_b, p->x_stride_l,
+            conv_bwd_cl_kernel<T, V, M2_ACT_SILU><<<grid, block, 0, st>>>(x, p->w, p->bias, dy, dx, part, l, C, p->x_stride_b, p->x_stride_l,
                                                                         p->y_stride_b, p->y_stride_l, p->dx_stride_b, p->dx_stride_l, p->param_dtype);
         else
-            conv_bwd_cl_kernel<T, M2_ACT_NONE><<<grid, block, 0, st>>>(x, p->w, p->bias, dy, dx, part, l, C, p->x_stride_b, p->x_stride_l,
+            conv_bwd_cl_kernel<T, V, M2_ACT_NONE><<<grid, block, 0, st>>>(x, p->w, p->bias, dy, dx, part, l, C, p->x_stride_b, p->x_stride_l,
                                                                         p->y_stride_b, p->y_stride_l, p->dx_stride_b, p->dx_stride_l, p->param_dtype);
         int rc = check_launch("conv1d_bwd");
         if (rc) return rc;

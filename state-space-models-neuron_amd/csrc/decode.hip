@@ -19,6 +19,8 @@
 namespace m2 {
 namespace {
 
+constexpr int kUP = 8;     // state rows a lane keeps in flight in the fast path
+
 __device__ __forceinline__ float ld_any(const void* p, int dt, int64_t i) {
     return dt == M2_F32 ? reinterpret_cast<const float*>(p)[i] : to_f32(reinterpret_cast<const bf16_t*>(p)[i]);
 }
@@ -48,6 +50,45 @@ decode_conv_kernel(const T* __restrict__ xBC, T* __restrict__ conv_state, const 
     (void)hist;
 }
 
+// bf16, k == 4, W in {3, 4}, Cx % 8 == 0: one thread owns 8 consecutive channels, whose W-column histories are
+// W*16 contiguous bytes; every access is a 16-byte vector.
+template <int W>
+__global__ void __launch_bounds__(256)
+decode_conv_vec_kernel(const bf16_t* __restrict__ xBC, bf16_t* __restrict__ conv_state, const void* __restrict__ w,
+                       const void* __restrict__ bias, float* __restrict__ act, int64_t nb, int64_t Cx, int64_t xsb, int pd,
+                       int activation) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;      // (b, c8)
+    const int64_t C8 = Cx / 8;
+    if (idx >= nb * C8) return;
+    const int64_t b = idx / C8, c0 = (idx % C8) * 8;
+    bf16_t* cs = conv_state + (b * Cx + c0) * W;
+    uint4 raw[W];
+#pragma unroll
+    for (int i = 0; i < W; ++i) raw[i] = reinterpret_cast<const uint4*>(cs)[i];
+    const uint4 xr = *reinterpret_cast<const uint4*>(xBC + b * xsb + c0);
+    const bf16_t* old = reinterpret_cast<const bf16_t*>(raw);                // [8 channels][W]
+    const bf16_t* xin = reinterpret_cast<const bf16_t*>(&xr);
+    uint4 nw[W];
+    bf16_t* nst = reinterpret_cast<bf16_t*>(nw);
+    float out[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        float z = bias ? ld_any(bias, pd, c0 + j) : 0.f;
+#pragma unroll
+        for (int i = 0; i < 3; ++i) z += ld_any(w, pd, (c0 + j) * 4 + i) * to_f32(old[j * W + (W - 3) + i]);
+        z += ld_any(w, pd, (c0 + j) * 4 + 3) * to_f32(xin[j]);
+#pragma unroll
+        for (int i = 0; i + 1 < W; ++i) nst[j * W + i] = old[j * W + i + 1];
+        nst[j * W + W - 1] = xin[j];
+        out[j] = activation == M2_ACT_SILU ? silu_f(z) : (activation == M2_ACT_RELU ? (z > 0.f ? z : 0.f) : z);
+    }
+#pragma unroll
+    for (int i = 0; i < W; ++i) reinterpret_cast<uint4*>(cs)[i] = nw[i];
+    float* ap = act + b * Cx + c0;
+    *reinterpret_cast<floatx4*>(ap) = floatx4{out[0], out[1], out[2], out[3]};
+    *reinterpret_cast<floatx4*>(ap + 4) = floatx4{out[4], out[5], out[6], out[7]};
+}
+
 // VEC = 4: n % 4 == 0, float4 accesses; VEC = 1: any n.
 // GL lanes (a power of two <= 64) share one state row; rows per pass = 256 / GL.
 template <typename T, int VEC>
@@ -68,6 +109,33 @@ decode_ssm_kernel(float* __restrict__ S, const float* __restrict__ act, const T*
     float* Sp = S + (b * nheads + h) * (int64_t)P * N;
     const int sub = tid % GL, rowi = tid / GL, rows_per_pass = 256 / GL;
     const int nv = N / VEC;
+    if (VEC == 4 && nv == GL && P % (rows_per_pass * kUP) == 0) {
+        // fast path (n = 4 * GL): each lane owns one float4 per row; kUP rows are loaded before any is used
+        const floatx4 bv = *reinterpret_cast<const floatx4*>(Ba + sub * 4);
+        const floatx4 cv = *reinterpret_cast<const floatx4*>(Ca + sub * 4);
+        for (int p0 = 0; p0 < P; p0 += rows_per_pass * kUP) {
+            floatx4 sv[kUP];
+            float xv[kUP];
+#pragma unroll
+            for (int u = 0; u < kUP; ++u) {
+                const int pp = p0 + u * rows_per_pass + rowi;
+                sv[u] = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(Sp + (int64_t)pp * N + sub * 4));
+                xv[u] = xa[pp];
+            }
+#pragma unroll
+            for (int u = 0; u < kUP; ++u) {
+                const int pp = p0 + u * rows_per_pass + rowi;
+                const float dx = dtv * xv[u];
+                float part = 0.f;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) { sv[u][q] = sv[u][q] * dA + dx * bv[q]; part += sv[u][q] * cv[q]; }
+                __builtin_nontemporal_store(sv[u], reinterpret_cast<floatx4*>(Sp + (int64_t)pp * N + sub * 4));
+                for (int off = GL >> 1; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+                if (sub == 0) y[b * ysb + h * P + pp] = from_f32<T>(part + Dh * xv[u]);
+            }
+        }
+        return;
+    }
     for (int p0 = 0; p0 < P; p0 += rows_per_pass) {
         const int pp = p0 + rowi;
         float part = 0.f, xv = 0.f;
@@ -126,12 +194,23 @@ extern "C" int m2_decode_step(const m2_decode_params* p, void* stream) {
     const int vec = (p->dstate % 4 == 0 && (p->nheads * p->headdim) % 4 == 0 && Cx % 4 == 0) ? 4 : 1;
     int GL = 1;
     while (GL < 64 && GL < p->dstate / vec) GL <<= 1;
+    const bool vec_conv = p->dtype == M2_BF16 && p->k == 4 && (p->W == 3 || p->W == 4) && Cx % 8 == 0 &&
+                          p->xBC_stride_b % 8 == 0 && aligned16(p->xBC) && aligned16(p->conv_state);
+    if (vec_conv) {
+        const unsigned blocks = (unsigned)ceil_div(p->batch * (Cx / 8), (int64_t)256);
+        const bf16_t* xb = static_cast<const bf16_t*>(p->xBC);
+        bf16_t* csb = static_cast<bf16_t*>(p->conv_state);
+        if (p->W == 3) decode_conv_vec_kernel<3><<<blocks, 256, 0, st>>>(xb, csb, p->conv_w, p->conv_b, act, p->batch, Cx, p->xBC_stride_b, p->param_dtype, p->activation);
+        else decode_conv_vec_kernel<4><<<blocks, 256, 0, st>>>(xb, csb, p->conv_w, p->conv_b, act, p->batch, Cx, p->xBC_stride_b, p->param_dtype, p->activation);
+        int rc = check_launch("decode_conv_vec_kernel");
+        if (rc) return rc;
+    }
     M2_DISPATCH_DTYPE(p->dtype, T, {
-        decode_conv_kernel<T><<<(unsigned)ceil_div(p->batch * Cx, (int64_t)256), 256, 0, st>>>(
+        if (!vec_conv) decode_conv_kernel<T><<<(unsigned)ceil_div(p->batch * Cx, (int64_t)256), 256, 0, st>>>(
             static_cast<const T*>(p->xBC), static_cast<T*>(p->conv_state), p->conv_w, p->conv_b, act, p->batch, Cx, p->k, p->W,
             p->xBC_stride_b, p->param_dtype, p->activation);
-        int rc = check_launch("decode_conv_kernel");
-        if (rc) return rc;
+        int rc2 = check_launch("decode_conv_kernel");
+        if (rc2) return rc2;
         dim3 grid((unsigned)p->nheads, (unsigned)p->batch);
         if (vec == 4)
             decode_ssm_kernel<T, 4><<<grid, 256, 0, st>>>(p->S, act, static_cast<const T*>(p->dt), p->A, p->D, static_cast<T*>(p->y),

@@ -9,7 +9,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmamba2_hip.so")
+# M2_LIB overrides the library path (used to compare builds of the same ABI)
+LIB_PATH = os.environ.get("M2_LIB") or os.path.join(_HERE, "libmamba2_hip.so")
 
 M2_F32, M2_BF16 = 0, 1
 ACT = {None: 0, "identity": 0, "silu": 1, "swish": 1, "relu": 2}
