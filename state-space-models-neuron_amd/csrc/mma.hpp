@@ -5,7 +5,7 @@
 // 16-byte ds_read (bf16) and the two operands use the same code path.
 //
 //   bf16: v_mfma_f32_32x32x16_bf16   lane -> row (lane & 31), k = 8 * (lane >> 5) + 0..7
-//   fp32: v_mfma_f32_32x32x2_f32     lane -> row (lane & 31), k = (lane >> 5)
+//   fp32: v_mfma_f32_32x32x2_f32     eight steps per 16 k, same lane -> (row, k) assignment (see Frag)
 //   accumulator (both): 16 floats per lane; register v of lane holds
 //        column  (lane & 31),   row  8 * (v >> 2) + 4 * (lane >> 5) + (v & 3)
 #pragma once
@@ -36,44 +36,66 @@ __device__ __forceinline__ void acc_zero(floatx16 (&acc)[BM][BN]) {
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 }
 
-// One wave: acc[i][j] (32x32 blocks) += A[rows i*32.., k0:k1] * Bt[rows j*32.., k0:k1]^T.
-// A points at the first of this wave's BM*32 rows, Bt at the first of its BN*32 rows.
-// k0, k1 multiples of 16.
-template <int BM, int BN>
-__device__ __forceinline__ void wave_mma(floatx16 (&acc)[BM][BN], const bf16_t* __restrict__ A, int lda,
-                                         const bf16_t* __restrict__ Bt, int ldb, int k0, int k1) {
+// A fragment is the slice of an MFMA operand one lane owns for a 16-wide k step: 8 CONSECUTIVE k values,
+// k = k0 + 8 * (lane >> 5) + 0..7, of row (lane & 31).  For bf16 this is the register layout of
+// v_mfma_f32_32x32x16_bf16.  For fp32 the same 8 values are fed to eight v_mfma_f32_32x32x2_f32 (element s of
+// both operands in step s); the hardware would pair k = 2s + (lane >> 5), but a contraction does not care in
+// which order k is visited as long as A and B agree, and the contiguous form needs two 16-byte reads
+// instead of eight scalar ones.
+template <typename T> struct Frag;
+template <> struct Frag<bf16_t> { bf16x8 v; };
+template <> struct Frag<float> { float v[8]; };
+
+__device__ __forceinline__ Frag<bf16_t> load_frag(const bf16_t* __restrict__ p) {
+    Frag<bf16_t> f;
+    f.v = *reinterpret_cast<const bf16x8*>(p);
+    return f;
+}
+__device__ __forceinline__ Frag<float> load_frag(const float* __restrict__ p) {
+    Frag<float> f;
+    const floatx4 a = *reinterpret_cast<const floatx4*>(p), b = *reinterpret_cast<const floatx4*>(p + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { f.v[i] = a[i]; f.v[4 + i] = b[i]; }
+    return f;
+}
+__device__ __forceinline__ void mma_frag(floatx16& acc, const Frag<bf16_t>& a, const Frag<bf16_t>& b) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, acc, 0, 0, 0);
+}
+__device__ __forceinline__ void mma_frag(floatx16& acc, const Frag<float>& a, const Frag<float>& b) {
+#pragma unroll
+    for (int s = 0; s < 8; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[s], b.v[s], acc, 0, 0, 0);
+}
+// element-wise scale of a fragment by 8 fp32 factors (one per k), result rounded to the operand type
+__device__ __forceinline__ Frag<bf16_t> scale_frag(const Frag<bf16_t>& a, const float (&f)[8]) {
+    Frag<bf16_t> r;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r.v[i] = (bf16_t)((float)a.v[i] * f[i]);
+    return r;
+}
+__device__ __forceinline__ Frag<float> scale_frag(const Frag<float>& a, const float (&f)[8]) {
+    Frag<float> r;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r.v[i] = a.v[i] * f[i];
+    return r;
+}
+
+// One wave: acc[i][j] (32x32 blocks) += A[rows i*32.., k0:k1] * Bt[rows j*32.., k0:k1]^T, operands in LDS.
+// A points at the first of this wave's BM*32 rows, Bt at the first of its BN*32 rows.  k0, k1 multiples of 16.
+template <int BM, int BN, typename T>
+__device__ __forceinline__ void wave_mma(floatx16 (&acc)[BM][BN], const T* __restrict__ A, int lda,
+                                         const T* __restrict__ Bt, int ldb, int k0, int k1) {
     const int lane = threadIdx.x & 63;
     const int r = lane & 31, kh = (lane >> 5) * 8;
     for (int k = k0; k < k1; k += 16) {
-        bf16x8 a[BM], b[BN];
+        Frag<T> a[BM], b[BN];
 #pragma unroll
-        for (int i = 0; i < BM; ++i) a[i] = *reinterpret_cast<const bf16x8*>(A + (i * 32 + r) * lda + k + kh);
+        for (int i = 0; i < BM; ++i) a[i] = load_frag(A + (i * 32 + r) * lda + k + kh);
 #pragma unroll
-        for (int j = 0; j < BN; ++j) b[j] = *reinterpret_cast<const bf16x8*>(Bt + (j * 32 + r) * ldb + k + kh);
-#pragma unroll
-        for (int i = 0; i < BM; ++i)
-#pragma unroll
-            for (int j = 0; j < BN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
-    }
-}
-
-template <int BM, int BN>
-__device__ __forceinline__ void wave_mma(floatx16 (&acc)[BM][BN], const float* __restrict__ A, int lda,
-                                         const float* __restrict__ Bt, int ldb, int k0, int k1) {
-    const int lane = threadIdx.x & 63;
-    const int r = lane & 31, kh = lane >> 5;
-    for (int k = k0; k < k1; k += 2) {
-        float a[BM], b[BN];
-#pragma unroll
-        for (int i = 0; i < BM; ++i) a[i] = A[(i * 32 + r) * lda + k + kh];
-#pragma unroll
-        for (int j = 0; j < BN; ++j) b[j] = Bt[(j * 32 + r) * ldb + k + kh];
+        for (int j = 0; j < BN; ++j) b[j] = load_frag(Bt + (j * 32 + r) * ldb + k + kh);
 #pragma unroll
         for (int i = 0; i < BM; ++i)
 #pragma unroll
-            for (int j = 0; j < BN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < BN; ++j) mma_frag(acc[i][j], a[i], b[j]);
     }
 }
 
@@ -89,6 +111,17 @@ __device__ __forceinline__ void stage_rows(T* __restrict__ s, int ld, const T* _
     constexpr int VPR = COLS / V;
     constexpr int TOTAL = ROWS * VPR;
     static_assert(COLS % V == 0, "tile width must be a multiple of the vector width");
+    if (!SCALE) {
+        // plain copy: 16 bytes stay 16 bytes, no conversion
+#pragma unroll 4
+        for (int e = tid; e < TOTAL; e += NT) {
+            const int r = e / VPR, cv = e % VPR;
+            uint4 raw = uint4{0u, 0u, 0u, 0u};
+            if (r < valid) raw = *reinterpret_cast<const uint4*>(g + (int64_t)r * gstride + cv * V);
+            *reinterpret_cast<uint4*>(s + r * ld + cv * V) = raw;
+        }
+        return;
+    }
 #pragma unroll 4
     for (int e = tid; e < TOTAL; e += NT) {
         const int r = e / VPR, cv = e % VPR;
@@ -116,6 +149,18 @@ __device__ __forceinline__ void stage_transposed(T* __restrict__ s, int ld, cons
     constexpr int VPR = COLS / V;
     constexpr int TOTAL = ROWS * VPR;
     static_assert(COLS % V == 0, "tile width must be a multiple of the vector width");
+    if (!SCALE) {
+#pragma unroll 4
+        for (int e = tid; e < TOTAL; e += NT) {
+            const int cv = e / ROWS, r = e % ROWS;
+            uint4 raw = uint4{0u, 0u, 0u, 0u};
+            if (r < valid) raw = *reinterpret_cast<const uint4*>(g + (int64_t)r * gstride + cv * V);
+            const T* el = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+            for (int i = 0; i < V; ++i) s[(cv * V + i) * ld + r] = el[i];
+        }
+        return;
+    }
 #pragma unroll 4
     for (int e = tid; e < TOTAL; e += NT) {
         // consecutive threads take consecutive tokens of the same channel vector: the LDS writes of a
@@ -132,6 +177,62 @@ __device__ __forceinline__ void stage_transposed(T* __restrict__ s, int ld, cons
 #pragma unroll
         for (int i = 0; i < V; ++i) s[(cv * V + i) * ld + r] = from_f32<T>(SCALE ? v[i] * sc : v[i]);
     }
+}
+
+// Sum of v over the 32 lanes that share (lane >> 5), for 16 values at once (the 16 accumulator rows of a lane),
+// by a butterfly reduce-scatter: 16 cross-lane moves instead of 80.  On return every lane holds ONE total:
+// that of register index  r = 8*b4 + 4*b3 + 2*b2 + b1  (b_k = bit k of lane), i.e. of accumulator row
+// acc_row(lane, r); lanes differing only in bit 0 hold the same total.
+__device__ __forceinline__ float half_wave_reduce16(float (&v)[16], int* reg_index) {
+    const int lane = threadIdx.x & 63;
+    const bool b4 = lane & 16, b3 = lane & 8, b2 = lane & 4, b1 = lane & 2;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const float keep = b4 ? v[k + 8] : v[k], send = b4 ? v[k] : v[k + 8];
+        v[k] = keep + __shfl_xor(send, 16, 64);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float keep = b3 ? v[k + 4] : v[k], send = b3 ? v[k] : v[k + 4];
+        v[k] = keep + __shfl_xor(send, 8, 64);
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const float keep = b2 ? v[k + 2] : v[k], send = b2 ? v[k] : v[k + 2];
+        v[k] = keep + __shfl_xor(send, 4, 64);
+    }
+    {
+        const float keep = b1 ? v[1] : v[0], send = b1 ? v[0] : v[1];
+        v[0] = keep + __shfl_xor(send, 2, 64);
+    }
+    v[0] += __shfl_xor(v[0], 1, 64);
+    *reg_index = (b4 ? 8 : 0) + (b3 ? 4 : 0) + (b2 ? 2 : 0) + (b1 ? 1 : 0);
+    return v[0];
+}
+
+// Wave-private chunk cumulative sum: every wave computes l for all 128 tokens by itself (lane holds tokens
+// `lane` and `lane + 64`), so no block barrier is needed.  Tokens >= valid behave as dt = 0.
+template <typename T>
+__device__ __forceinline__ void wave_chunk_cumsum(const void* __restrict__ dt, int dt_f32, int64_t off, int64_t stride_l,
+                                                  int valid, float A, float& l0, float& l1, float& d0, float& d1) {
+    const int lane = threadIdx.x & 63;
+    d0 = 0.f; d1 = 0.f;
+    if (dt_f32) {
+        const float* p = static_cast<const float*>(dt) + off;
+        if (lane < valid) d0 = p[(int64_t)lane * stride_l];
+        if (lane + 64 < valid) d1 = p[(int64_t)(lane + 64) * stride_l];
+    } else {
+        const T* p = static_cast<const T*>(dt) + off;
+        if (lane < valid) d0 = to_f32(p[(int64_t)lane * stride_l]);
+        if (lane + 64 < valid) d1 = to_f32(p[(int64_t)(lane + 64) * stride_l]);
+    }
+    l0 = A * d0; l1 = A * d1;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const float n0 = __shfl_up(l0, o, 64), n1 = __shfl_up(l1, o, 64);
+        if (lane >= o) { l0 += n0; l1 += n1; }
+    }
+    l1 += __shfl(l0, 63, 64);
 }
 
 // Inclusive cumulative sum l[t] = sum_{s<=t} A * dt[s] over one chunk (kQ = 128 tokens), in fp32.

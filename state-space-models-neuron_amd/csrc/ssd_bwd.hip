@@ -26,402 +26,330 @@
 //   cb_kernel, chunk_state_kernel, state_scan_kernel          recompute G, S_prev, final state
 //   chunk_state_kernel<DSTATE>                                local dS contributions  e^{l} dy^T C
 //   state_scan_kernel<REVERSE>                                dS per chunk, <dS, S_new>, d initial state
-//   group_grad_kernel      per (b, chunk, group, head slice)  partial dB, dC (heads reduced in registers), dl per head
-//   dx_kernel              per (b, chunk, head)               dx, ddt, partial dA, dD
-//   bc_reduce_kernel, ad_reduce_kernel                        sum the partials (fixed order, no atomics)
+//   dg_kernel              per (b, chunk, group, head slice)  partial dG (heads reduced in registers), dl_diag per head
+//   off_kernel<C>, <B>     per (b, chunk, group, head slice)  partial state parts of dC / dB, dl_c per head
+//   diag_off_kernel<bwd>   per (b, chunk, group, head slice)  dx, ddt, partial dA, dD (dl assembled here)
+//   bc_final_kernel        per (b, chunk, group)              dC = dG B + dCoff, dB = dG^T C + dBoff
+//   ad_reduce_kernel                                          dA, dD (fixed order, no atomics)
 #include "ssd_host.hpp"
 
 namespace m2 {
 namespace {
 
-__device__ __forceinline__ float half_wave_sum(float v) {   // sum over the 32 lanes sharing (lane >> 5)
-#pragma unroll
-    for (int off = 16; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
-
 // ------------------------------------------------------------------------------------------
-// grid (nchunks, nheads, batch), 256 threads; wave w owns token rows 32w..32w+31.
-template <typename T, int P, int N>
-__global__ void __launch_bounds__(256)
-dx_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f32, const float* __restrict__ A,
-          const T* __restrict__ Bm, const float* __restrict__ D, const float* __restrict__ G,
-          const float* __restrict__ dl, const T* __restrict__ dY, const T* __restrict__ dprev, const float* __restrict__ dlam,
-          T* __restrict__ dX, void* __restrict__ ddt, float* __restrict__ dAp, float* __restrict__ dDp,
-          int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks,
-          int64_t Xsb, int64_t Xsl, int64_t Xsh, int64_t dtsb, int64_t dtsl,
-          int64_t Bsb, int64_t Bsl, int64_t Bsg,
-          int64_t dYsb, int64_t dYsl, int64_t dYsh, int64_t dXsb, int64_t dXsl, int64_t dXsh,
-          int64_t ddtsb, int64_t ddtsl) {
-    constexpr int LDN = lds_ld<T>(N);
-    constexpr int LDQ = lds_ld<T>(kQ);
-    constexpr int BN = P / 32;
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    float* s_l = reinterpret_cast<float*>(smem_raw);
-    float* s_dt = s_l + kQ;
-    float* s_w = s_dt + kQ;
-    float* s_dir = s_w + kQ;
-    float* s_tmp = s_dir + kQ;                     // 4 floats
-    float* s_red = s_tmp + 4;                      // 8 floats
-    T* buf = reinterpret_cast<T*>(s_red + 8);
-    T* sB = buf;                                   // phase 1: [kQ][LDN]
-    T* sdS = buf + kQ * LDN;                       //          [P][LDN]
-    T* sMt = buf;                                  // phase 2: [kQ][LDQ]   Mt[j][i]
-    T* sdYt = buf + kQ * LDQ;                      //          [P][LDQ]
+// dG partial and the diagonal part of the decay gradient.
+// grid (nchunks, ngroups * nslices, batch), 512 threads (8 waves).  Wave w owns the 32x32 blocks of the
+// [kQ][kQ] tile with block-row rb = w >> 1 and block-columns cb0 = 2 (w & 1), cb0 + 1.
+//   per head:  P = dY X^T  (MFMA, K = headdim);   dG^h[i][j] = e^{l_i - l_j} dt_j P[i][j]   (i >= j)
+//              dG += dG^h;    pr = dG^h o G;   dl_diag[i] = sum_j pr[i][j] - sum_i' pr[i'][i]
+// Row and column sums come from the same fp32 products, so pairs inside a suffix cancel exactly.
+template <typename T, int P>
+constexpr bool dg_g_in_lds() { return (size_t)14 * kQ * sizeof(float) + ((size_t)2 * kQ * lds_ld<T>(P) + (size_t)kQ * lds_ld<T>(kQ)) * sizeof(T) <= 150 * 1024; }
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int64_t c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    const int64_t g = h / (nheads / ngroups);
-    const int64_t t0 = c * kQ;
-    const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
-    const float Ah = A[h];
-
-    chunk_cumsum_any<T>(dt, dt_f32, b * dtsb + t0 * dtsl + h, dtsl, valid, Ah, s_l, s_dt, s_tmp, tid);
-    const float Lam = s_l[kQ - 1];
-
-    // ---- phase 1: acc[j][p] = e^{Lam-l_j} * sum_n B[j][n] dS[p][n]
-    const int64_t tile = ((b * nchunks + c) * nheads + h) * (int64_t)(P * N);
-    stage_rows<T, kQ, N, 256, false>(sB, LDN, Bm + b * Bsb + t0 * Bsl + g * Bsg, Bsl, valid, nullptr, tid);
-    stage_rows<T, P, N, 256, false>(sdS, LDN, dprev + tile, N, P, nullptr, tid);
-    __syncthreads();
-    floatx16 acc[1][BN];
-    acc_zero(acc);
-    wave_mma<1, BN>(acc, sB + wave * 32 * LDN, LDN, sdS, LDN, 0, N);
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const float e = __expf(Lam - s_l[wave * 32 + acc_row(lane, v)]);
-#pragma unroll
-        for (int j = 0; j < BN; ++j) acc[0][j][v] *= e;
-    }
-    __syncthreads();
-
-    // ---- phase 2: acc[j][p] += sum_{i>=j} (e^{l_i-l_j} G[i][j]) dy[i][p]
-    const float* Gp = G + ((b * nchunks + c) * ngroups + g) * (int64_t)(kQ * kQ);
-    for (int e = tid; e < kQ * (kQ / 4); e += 256) {
-        const int i = e / (kQ / 4), j4 = (e % (kQ / 4)) * 4;
-        if ((j4 >> 5) > (i >> 5)) continue;
-        const floatx4 g4 = *reinterpret_cast<const floatx4*>(Gp + i * kQ + j4);
-        const float li = s_l[i];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int j = j4 + q;
-            const float m = (j <= i) ? __expf(li - s_l[j]) * g4[q] : 0.f;
-            sMt[j * LDQ + i] = from_f32<T>(m);
-        }
-    }
-    stage_transposed<T, kQ, P, 256, false>(sdYt, LDQ, dY + b * dYsb + t0 * dYsl + h * dYsh, dYsl, valid, nullptr, tid);
-    __syncthreads();
-    wave_mma<1, BN>(acc, sMt + wave * 32 * LDQ, LDQ, sdYt, LDQ, wave * 32, kQ);
-
-    // ---- epilogue
-    const float Dh = D ? D[h] : 0.f;
-    const T* Xp = X + b * Xsb + t0 * Xsl + h * Xsh;
-    T* dXp = dX + b * dXsb + t0 * dXsl + h * dXsh;
-    float dD_loc = 0.f;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const int row = wave * 32 + acc_row(lane, v);
-        float edir = 0.f;
-        if (row < valid) {
-            const float dtj = s_dt[row];
-#pragma unroll
-            for (int j = 0; j < BN; ++j) {
-                const int col = j * 32 + acc_col(lane);
-                const float xv = to_f32(Xp[(int64_t)row * Xsl + col]);
-                const float gy = to_f32(sdYt[col * LDQ + row]);
-                const float dxd = acc[0][j][v];
-                dXp[(int64_t)row * dXsl + col] = from_f32<T>(dtj * dxd + Dh * gy);
-                edir += dxd * xv;
-                dD_loc += gy * xv;
-            }
-        }
-        edir = half_wave_sum(edir);
-        if ((lane & 31) == 0) s_dir[row] = edir;
-    }
-    dD_loc = warp_sum(dD_loc);
-    if (lane == 0) s_red[wave] = dD_loc;
-    __syncthreads();
-
-    // ---- da_j = (suffix sum of dl inside the chunk) + <dS, S_new>;  ddt, partial dA, partial dD
-    float da_dt = 0.f;
-    if (tid < kQ) {
-        const int j = kQ - 1 - tid;                // thread t scans token Q-1-t: prefix over t == suffix over j
-        float s = dl[((b * nheads + h) * nchunks + c) * kQ + j];
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const float nb = __shfl_up(s, off, 64);
-            if (lane >= off) s += nb;
-        }
-        if (tid == 63) s_tmp[1] = s;
-        s_w[j] = s;                                // own slot only; completed after the barrier
-    }
-    __syncthreads();
-    if (tid < kQ) {
-        const int j = kQ - 1 - tid;
-        float s = s_w[j];
-        if (tid >= 64) s += s_tmp[1];
-        const float da = s + dlam[(b * nheads + h) * nchunks + c];
-        if (j < valid) {
-            const float val = Ah * da + s_dir[j];
-            const int64_t o = b * ddtsb + (t0 + j) * ddtsl + h;
-            if (dt_f32) static_cast<float*>(ddt)[o] = val;
-            else static_cast<T*>(ddt)[o] = from_f32<T>(val);
-            da_dt = da * s_dt[j];
-        }
-    }
-    da_dt = warp_sum(da_dt);
-    if (lane == 0) s_red[4 + wave] = da_dt;
-    __syncthreads();
-    if (tid == 0) {
-        const int64_t o = (b * nheads + h) * nchunks + c;
-        dAp[o] = s_red[4] + s_red[5] + s_red[6] + s_red[7];
-        dDp[o] = s_red[0] + s_red[1] + s_red[2] + s_red[3];
-    }
-}
-
-// ------------------------------------------------------------------------------------------
-// grid (nchunks, ngroups * nslices, batch), 512 threads (8 waves).
-// Wave w owns 32x32 blocks: row block (w >> 1), column blocks (w & 1) * NB + {0..NB-1}.
-template <typename T, int P, int N>
-__global__ void __launch_bounds__(512)
-group_grad_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f32, const float* __restrict__ A,
-                  const T* __restrict__ Bm, const T* __restrict__ Cm, const T* __restrict__ dY,
-                  const T* __restrict__ Sprev, const T* __restrict__ dprev, const float* __restrict__ G,
-                  float* __restrict__ dBp, float* __restrict__ dCp, float* __restrict__ dl,
-                  int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks, int64_t nslices, int64_t hps,
-                  int64_t Xsb, int64_t Xsl, int64_t Xsh, int64_t dtsb, int64_t dtsl,
-                  int64_t Bsb, int64_t Bsl, int64_t Bsg, int64_t Csb, int64_t Csl, int64_t Csg,
-                  int64_t dYsb, int64_t dYsl, int64_t dYsh) {
+template <typename T, int P>
+__global__ void __launch_bounds__(512, 2)
+dg_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f32, const float* __restrict__ A,
+          const T* __restrict__ dY, const T* __restrict__ Gm, float* __restrict__ dGp, float* __restrict__ dl_diag,
+          int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks, int64_t nslices, int64_t hps,
+          int64_t Xsb, int64_t Xsl, int64_t Xsh, int64_t dtsb, int64_t dtsl, int64_t dYsb, int64_t dYsl, int64_t dYsh) {
     constexpr int LDP = lds_ld<T>(P);
     constexpr int LDQ = lds_ld<T>(kQ);
-    constexpr int NB = N / 64;                    // column blocks per wave for [Q][N] outputs
-    constexpr int SZ1 = 2 * kQ * LDP, SZ2 = (kQ + N) * LDQ, SZ3 = (kQ + N) * LDP;
-    constexpr int SZ = SZ1 > SZ2 ? (SZ1 > SZ3 ? SZ1 : SZ3) : (SZ2 > SZ3 ? SZ2 : SZ3);
-    (void)SZ;
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    float* s_l = reinterpret_cast<float*>(smem_raw);
-    float* s_dt = s_l + kQ;
-    float* s_e = s_dt + kQ;                        // e^{l_i}
-    float* s_d = s_e + kQ;                         // dt_j e^{Lam - l_j}
-    float* s_tmp = s_d + kQ;                       // 4 floats
-    float* s_rs = s_tmp + 4;                       // [2][kQ] row sums of dG^h o G   (one slot per column half)
-    float* s_cs = s_rs + 2 * kQ;                   // [4][kQ] column sums of dG^h o G (one slot per row block)
-    float* s_rc = s_cs + 4 * kQ;                   // [2][kQ] C_i . dCoff_i^h
-    float* s_rb = s_rc + 2 * kQ;                   // [2][kQ] B_j . dBoff_j^h
-    T* buf = reinterpret_cast<T*>(s_rb + 2 * kQ);
-    T* sA = buf;                                   // first tile  [kQ][LDP]  (or [kQ][LDQ] in the final steps)
-    T* sT = buf + kQ * LDP;                        // second tile [kQ or N][LDP]
-    T* sA2 = buf;                                  // final: [kQ][LDQ]
-    T* sT2 = buf + kQ * LDQ;                       // final: [N][LDQ]
+    float* wtab = reinterpret_cast<float*>(smem_raw);      // [8 waves][kQ]  l (wave-private)
+    float* s_rs = wtab + 8 * kQ;                           // [2][kQ]
+    float* s_cs = s_rs + 2 * kQ;                           // [4][kQ]
+    T* sA = reinterpret_cast<T*>(s_cs + 4 * kQ);           // dY [kQ][LDP]
+    T* sT = sA + kQ * LDP;                                 // X  [kQ][LDP]
+    T* sG = sT + kQ * LDP;                                 // G  [kQ][LDQ]  (blocks above the diagonal are never read)
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 31, half = lane >> 5;
     const int64_t c = blockIdx.x, b = blockIdx.z;
     const int64_t g = blockIdx.y / nslices, slice = blockIdx.y % nslices;
     const int64_t hpg = nheads / ngroups;
     const int64_t t0 = c * kQ;
     const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
-    const int rb = wave >> 1, cb0 = (wave & 1) * 2;       // [Q][Q] blocks: 2 per wave
-    const int nb0 = (wave & 1) * NB;                        // [Q][N] blocks: NB per wave
+    const int rb = wave >> 1, cb0 = (wave & 1) * 2;
+    const bool active = cb0 <= rb;
+    float* wl = wtab + wave * kQ;
 
-    floatx16 dG[1][2], dC[1][NB], dB[1][NB];
-    acc_zero(dG); acc_zero(dC); acc_zero(dB);
+    // causal-masked G of this (chunk, group), shared by all heads: staged once
+    constexpr bool G_LDS = dg_g_in_lds<T, P>();
+    const T* Gg = Gm + ((b * nchunks + c) * ngroups + g) * (int64_t)(kQ * kQ);
+    if (G_LDS) stage_rows<T, kQ, kQ, 512, false>(sG, LDQ, Gg, kQ, kQ, nullptr, tid);
+    floatx16 dG[1][2];
+    acc_zero(dG);
 
     for (int64_t hh = 0; hh < hps; ++hh) {
         const int64_t h = g * hpg + slice * hps + hh;
-        chunk_cumsum_any<T>(dt, dt_f32, b * dtsb + t0 * dtsl + h, dtsl, valid, A[h], s_l, s_dt, s_tmp, tid);
-        const float Lam = s_l[kQ - 1];
-        if (tid < kQ) { s_e[tid] = __expf(s_l[tid]); s_d[tid] = s_dt[tid] * __expf(Lam - s_l[tid]); }
-        const T* Xp = X + b * Xsb + t0 * Xsl + h * Xsh;
-        const T* dYp = dY + b * dYsb + t0 * dYsl + h * dYsh;
-        const int64_t tile = ((b * nchunks + c) * nheads + h) * (int64_t)(P * N);
+        float l0, l1, d0, d1;
+        wave_chunk_cumsum<T>(dt, dt_f32, b * dtsb + t0 * dtsl + h, dtsl, valid, A[h], l0, l1, d0, d1);
+        wl[lane] = l0; wl[lane + 64] = l1;
+        const float l_first = rb < 2 ? __shfl(l0, rb * 32, 64) : __shfl(l1, rb * 32 - 64, 64);
+        const float l_last = rb < 2 ? __shfl(l0, rb * 32 + 31, 64) : __shfl(l1, rb * 32 + 31 - 64, 64);
+        const bool fast = (l_first - l_last) < kMaxRange;
+        // column-side values of this lane's two columns j = (cb0 + jb) * 32 + r
+        float lj[2], dtj[2], vj[2];
+#pragma unroll
+        for (int jb = 0; jb < 2; ++jb) {
+            const int src = jb * 32 + r;
+            lj[jb] = cb0 == 0 ? __shfl(l0, src, 64) : __shfl(l1, src, 64);
+            dtj[jb] = cb0 == 0 ? __shfl(d0, src, 64) : __shfl(d1, src, 64);
+            vj[jb] = (cb0 + jb <= rb) ? __expf(fminf(l_first - lj[jb], kMaxRange)) * dtj[jb] : 0.f;
+        }
 
-        // ---- A: dG[i][j] += e^{l_i-l_j} dt_j (dy_i . x_j),  i >= j
-        stage_rows<T, kQ, P, 512, false>(sA, LDP, dYp, dYsl, valid, nullptr, tid);
-        stage_rows<T, kQ, P, 512, false>(sT, LDP, Xp, Xsl, valid, nullptr, tid);
+        __syncthreads();      // previous head: tiles consumed, s_rs / s_cs consumed
+        stage_rows<T, kQ, P, 512, false>(sA, LDP, dY + b * dYsb + t0 * dYsl + h * dYsh, dYsl, valid, nullptr, tid);
+        stage_rows<T, kQ, P, 512, false>(sT, LDP, X + b * Xsb + t0 * Xsl + h * Xsh, Xsl, valid, nullptr, tid);
         __syncthreads();
-        const float* Gp = G + ((b * nchunks + c) * ngroups + g) * (int64_t)(kQ * kQ);
-        {
-            floatx16 pa[1][2];
-            acc_zero(pa);
-            float rsum[16], csum[2];
+
+        float rsum[16], csum[2] = {0.f, 0.f};
 #pragma unroll
-            for (int v = 0; v < 16; ++v) rsum[v] = 0.f;
-            csum[0] = csum[1] = 0.f;
-            if (cb0 <= rb) {
-                wave_mma<1, 2>(pa, sA + rb * 32 * LDP, LDP, sT + cb0 * 32 * LDP, LDP, 0, P);
-#pragma unroll
-                for (int jb = 0; jb < 2; ++jb) {
-                    if (cb0 + jb > rb) continue;
-                    const int j = (cb0 + jb) * 32 + acc_col(lane);
-                    const float lj = s_l[j], dtj = s_dt[j];
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int i = rb * 32 + acc_row(lane, v);
-                        if (i >= j) {
-                            const float dgh = __expf(s_l[i] - lj) * dtj * pa[0][jb][v];
-                            dG[0][jb][v] += dgh;
-                            const float pr = dgh * Gp[i * kQ + j];
-                            rsum[v] += pr;
-                            csum[jb] += pr;
-                        }
-                    }
-                }
-            }
-            // row sums: over the 32 lanes of a half wave (columns) -> slot (wave & 1) of row i
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const float r = half_wave_sum(rsum[v]);
-                if ((lane & 31) == 0) s_rs[(wave & 1) * kQ + rb * 32 + acc_row(lane, v)] = r;
-            }
-            // column sums: over this lane's 16 rows, then the other half wave -> slot rb of column j
+        for (int v = 0; v < 16; ++v) rsum[v] = 0.f;
+        if (active) {
 #pragma unroll
             for (int jb = 0; jb < 2; ++jb) {
-                const float cs = csum[jb] + __shfl_xor(csum[jb], 32, 64);
-                if (lane < 32) s_cs[rb * kQ + (cb0 + jb) * 32 + lane] = cs;
-            }
-        }
-        __syncthreads();
-
-        // ---- B: dC[i][n] += e^{l_i} sum_p dy[i][p] S_prev[p][n]     (dy tile still in sA; row scale applied in fp32)
-        stage_transposed<T, P, N, 512, false>(sT, LDP, Sprev + tile, N, P, nullptr, tid);
-        __syncthreads();
-        {
-            floatx16 tc[1][NB];
-            acc_zero(tc);
-            wave_mma<1, NB>(tc, sA + rb * 32 * LDP, LDP, sT + nb0 * 32 * LDP, LDP, 0, P);
-            const T* Cg = Cm + b * Csb + t0 * Csl + g * Csg;
+                if (cb0 + jb > rb) continue;
+                floatx16 pa[1][1];
+                acc_zero(pa);
+                wave_mma<1, 1>(pa, sA + rb * 32 * LDP, LDP, sT + (cb0 + jb) * 32 * LDP, LDP, 0, P);
+                const int j = (cb0 + jb) * 32 + r;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int i = rb * 32 + acc_row(lane, v);
-                const float sc = s_e[i];
-                float r = 0.f;
-#pragma unroll
-                for (int jn = 0; jn < NB; ++jn) {
-                    const float t = tc[0][jn][v] * sc;
-                    dC[0][jn][v] += t;
-                    if (i < valid) r += t * to_f32(Cg[(int64_t)i * Csl + (nb0 + jn) * 32 + acc_col(lane)]);
+                for (int v = 0; v < 16; ++v) {
+                    const int i = rb * 32 + acc_row(lane, v);
+                    float w;
+                    if (fast) w = __expf(wl[i] - l_first) * vj[jb];            // u_i * v_j
+                    else w = __expf(fminf(wl[i] - lj[jb], 0.f)) * dtj[jb];
+                    const float dgh = (i >= j) ? w * pa[0][0][v] : 0.f;
+                    dG[0][jb][v] += dgh;
+                    const float pr = dgh * to_f32(G_LDS ? sG[i * LDQ + j] : Gg[i * kQ + j]);
+                    rsum[v] += pr;
+                    csum[jb] += pr;
                 }
-                r = half_wave_sum(r);
-                if ((lane & 31) == 0) s_rc[(wave & 1) * kQ + i] = r;
             }
         }
-        __syncthreads();
-
-        // ---- C: dB[j][n] += dt_j e^{Lam-l_j} sum_p x[j][p] dS[p][n]
-        stage_rows<T, kQ, P, 512, false>(sA, LDP, Xp, Xsl, valid, nullptr, tid);
-        stage_transposed<T, P, N, 512, false>(sT, LDP, dprev + tile, N, P, nullptr, tid);
-        __syncthreads();
-        {
-            floatx16 tb[1][NB];
-            acc_zero(tb);
-            wave_mma<1, NB>(tb, sA + rb * 32 * LDP, LDP, sT + nb0 * 32 * LDP, LDP, 0, P);
-            const T* Bg = Bm + b * Bsb + t0 * Bsl + g * Bsg;
+        int ri;
+        const float rtot = half_wave_reduce16(rsum, &ri);
+        if ((lane & 1) == 0) s_rs[(wave & 1) * kQ + rb * 32 + acc_row(lane, ri)] = rtot;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int j = rb * 32 + acc_row(lane, v);
-                const float sc = s_d[j];
-                float r = 0.f;
-#pragma unroll
-                for (int jn = 0; jn < NB; ++jn) {
-                    const float t = tb[0][jn][v] * sc;
-                    dB[0][jn][v] += t;
-                    if (j < valid) r += t * to_f32(Bg[(int64_t)j * Bsl + (nb0 + jn) * 32 + acc_col(lane)]);
-                }
-                r = half_wave_sum(r);
-                if ((lane & 31) == 0) s_rb[(wave & 1) * kQ + j] = r;
-            }
+        for (int jb = 0; jb < 2; ++jb) {
+            const float cs = csum[jb] + __shfl_xor(csum[jb], 32, 64);
+            if (lane < 32) s_cs[rb * kQ + (cb0 + jb) * 32 + lane] = cs;
         }
         __syncthreads();
-        // dl_t for this head: row role minus column role
         if (tid < kQ) {
             const float rs = s_rs[tid] + s_rs[kQ + tid];
             const float cs = s_cs[tid] + s_cs[kQ + tid] + s_cs[2 * kQ + tid] + s_cs[3 * kQ + tid];
-            const float rc = s_rc[tid] + s_rc[kQ + tid];
-            const float rbv = s_rb[tid] + s_rb[kQ + tid];
-            dl[((b * nheads + h) * nchunks + c) * kQ + tid] = rs - cs + rc - rbv;
+            dl_diag[((b * nheads + h) * nchunks + c) * kQ + tid] = rs - cs;
         }
     }
+    if (!active) return;
+    float* out = dGp + (((b * nchunks + c) * ngroups + g) * nslices + slice) * (int64_t)(kQ * kQ);
+#pragma unroll
+    for (int jb = 0; jb < 2; ++jb) {
+        if (cb0 + jb > rb) continue;
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            out[(rb * 32 + acc_row(lane, v)) * kQ + (cb0 + jb) * 32 + r] = dG[0][jb][v];
+    }
+}
 
-    const T* Bp = Bm + b * Bsb + t0 * Bsl + g * Bsg;
-    const T* Cp = Cm + b * Csb + t0 * Csl + g * Csg;
+// ------------------------------------------------------------------------------------------
+// Off-diagonal (state) parts of dC and dB, heads of a slice reduced in registers.
+// grid (nchunks, ngroups * nslices, batch), 512 threads.  Wave w owns rows rb = w >> 1 and state-column blocks
+// nb0 = (w & 1) * NB .. + NB - 1 of the [kQ][N] tile.
+//   SIDE_C:  dC[i][n] += e^{l_i} sum_p dy[i][p] S_prev[p][n];   dl_c[i] = C_i . (that head's contribution)
+//   SIDE_B:  dB[j][n] += dt_j e^{Lam - l_j} sum_p x[j][p] dS[p][n]
+// The row scale is applied in fp32 after the MFMA, so both operands are exact copies of the inputs.
+template <typename T, int P, int N>
+constexpr bool off_c_in_lds() { return (size_t)10 * kQ * sizeof(float) + ((size_t)(kQ + N) * lds_ld<T>(P) + (size_t)kQ * lds_ld<T>(N)) * sizeof(T) <= 150 * 1024; }
 
-    // The head-summed dG is rounded to the operand type only here.  For bf16 it is split into
-    // hi + lo (two MFMA passes) so that the group-level contractions see it at ~2^-17 relative.
+template <typename T, int P, int N, bool SIDE_C>
+__global__ void __launch_bounds__(512, SIDE_C ? 2 : 4)
+off_kernel(const T* __restrict__ Arow, int64_t Asb, int64_t Asl, int64_t Ash,      // dY (C side) or X (B side)
+           const void* __restrict__ dt, int dt_f32, const float* __restrict__ A,
+           const T* __restrict__ St,                                               // S_prev (C side) or dS (B side): [b][c][h][P][N]
+           const T* __restrict__ Cm, int64_t Csb, int64_t Csl, int64_t Csg,        // C side only
+           float* __restrict__ outp, float* __restrict__ dl_c,
+           int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks, int64_t nslices, int64_t hps,
+           int64_t dtsb, int64_t dtsl) {
+    constexpr int LDP = lds_ld<T>(P);
+    constexpr int NB = N / 64;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    float* wtab = reinterpret_cast<float*>(smem_raw);      // [8 waves][kQ]  row scale (wave-private)
+    float* s_rc = wtab + 8 * kQ;                           // [2][kQ]
+    T* sA = reinterpret_cast<T*>(s_rc + 2 * kQ);           // [kQ][LDP]
+    T* sT = sA + kQ * LDP;                                 // [N][LDP]   state tile transposed
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 31;
+    const int64_t c = blockIdx.x, b = blockIdx.z;
+    const int64_t g = blockIdx.y / nslices, slice = blockIdx.y % nslices;
+    const int64_t hpg = nheads / ngroups;
+    const int64_t t0 = c * kQ;
+    const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
+    const int rb = wave >> 1, nb0 = (wave & 1) * NB;
+    float* ws = wtab + wave * kQ;
+
+    constexpr int LDN = lds_ld<T>(N);
+    T* sC = sT + N * LDP;                                  // C side: C [kQ][LDN], staged once for all heads
+    constexpr bool C_LDS = off_c_in_lds<T, P, N>();
+    const T* Cgl = SIDE_C ? Cm + b * Csb + t0 * Csl + g * Csg : nullptr;
+    if (SIDE_C && C_LDS) stage_rows<T, kQ, N, 512, false>(sC, LDN, Cgl, Csl, valid, nullptr, tid);
+    floatx16 acc[1][NB];
+    acc_zero(acc);
+
+    for (int64_t hh = 0; hh < hps; ++hh) {
+        const int64_t h = g * hpg + slice * hps + hh;
+        float l0, l1, d0, d1;
+        wave_chunk_cumsum<T>(dt, dt_f32, b * dtsb + t0 * dtsl + h, dtsl, valid, A[h], l0, l1, d0, d1);
+        if (SIDE_C) { ws[lane] = __expf(l0); ws[lane + 64] = __expf(l1); }
+        else {
+            const float Lam = __shfl(l1, 63, 64);
+            ws[lane] = d0 * __expf(Lam - l0); ws[lane + 64] = d1 * __expf(Lam - l1);
+        }
+        const int64_t tile = ((b * nchunks + c) * nheads + h) * (int64_t)(P * N);
+        __syncthreads();
+        stage_rows<T, kQ, P, 512, false>(sA, LDP, Arow + b * Asb + t0 * Asl + h * Ash, Asl, valid, nullptr, tid);
+        stage_transposed<T, P, N, 512, false>(sT, LDP, St + tile, N, P, nullptr, tid);
+        __syncthreads();
+        float rcv[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) rcv[v] = 0.f;
+#pragma unroll
+        for (int jn = 0; jn < NB; ++jn) {
+            floatx16 tc[1][1];
+            acc_zero(tc);
+            wave_mma<1, 1>(tc, sA + rb * 32 * LDP, LDP, sT + (nb0 + jn) * 32 * LDP, LDP, 0, P);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float t = tc[0][0][v] * ws[rb * 32 + acc_row(lane, v)];
+                acc[0][jn][v] += t;
+                if (SIDE_C) {
+                    const int i = rb * 32 + acc_row(lane, v), n = (nb0 + jn) * 32 + r;
+                    const T cval = C_LDS ? sC[i * LDN + n] : (i < valid ? Cgl[(int64_t)i * Csl + n] : (T)0.f);
+                    rcv[v] += t * to_f32(cval);
+                }
+            }
+        }
+        if (SIDE_C) {
+            int ri;
+            const float tot = half_wave_reduce16(rcv, &ri);
+            if ((lane & 1) == 0) s_rc[(wave & 1) * kQ + rb * 32 + acc_row(lane, ri)] = tot;
+            __syncthreads();
+            if (tid < kQ) dl_c[((b * nheads + h) * nchunks + c) * kQ + tid] = s_rc[tid] + s_rc[kQ + tid];
+        }
+    }
+    float* out = outp + (((b * nchunks + c) * ngroups + g) * nslices + slice) * (int64_t)(kQ * N);
+#pragma unroll
+    for (int jn = 0; jn < NB; ++jn)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            out[(rb * 32 + acc_row(lane, v)) * N + (nb0 + jn) * 32 + r] = acc[0][jn][v];
+}
+
+// Sum of the per-slice partials (fixed order).  One thread per float4; `tile` floats per (group, slice) tile.
+__global__ void __launch_bounds__(256)
+slice_sum_kernel(const float* __restrict__ part, float* __restrict__ out, int64_t ngrp, int64_t nslices, int64_t tile) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t per = tile / 4;
+    if (idx >= ngrp * per) return;
+    const int64_t grp = idx / per, e = (idx % per) * 4;
+    floatx4 s = {0.f, 0.f, 0.f, 0.f};
+    for (int64_t sl = 0; sl < nslices; ++sl) s += *reinterpret_cast<const floatx4*>(part + (grp * nslices + sl) * tile + e);
+    *reinterpret_cast<floatx4*>(out + grp * tile + e) = s;
+}
+
+// ------------------------------------------------------------------------------------------
+// Group-level finish: dG = sum of the slice partials; dC = dG B + sum dCoff;  dB = dG^T C + sum dBoff.
+// grid (nchunks, ngroups, batch), 512 threads.  The head-summed dG is rounded to the operand type only here; for
+// bf16 it is split into hi + lo (two MFMA passes) so the contractions see it at ~2^-17 relative.
+template <typename T, int N>
+__global__ void __launch_bounds__(512)
+bc_final_kernel(const float* __restrict__ dGp, const float* __restrict__ dCp, const float* __restrict__ dBp,
+                const T* __restrict__ Bt, const T* __restrict__ Ct, T* __restrict__ dB, T* __restrict__ dC,
+                int64_t seqlen, int64_t ngroups, int64_t nchunks,
+                int64_t dBsb, int64_t dBsl, int64_t dBsg, int64_t dCsb, int64_t dCsl, int64_t dCsg) {
+    constexpr int LDQ = lds_ld<T>(kQ);
+    constexpr int NB = N / 64;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* sA2 = reinterpret_cast<T*>(smem_raw);       // [kQ][LDQ]  dG (or its transpose)
+    T* sT2 = sA2 + kQ * LDQ;                       // [N][LDQ]   Bt or Ct
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 31;
+    const int64_t c = blockIdx.x, g = blockIdx.y, b = blockIdx.z;
+    const int64_t t0 = c * kQ;
+    const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
+    const int rb = wave >> 1, cb0 = (wave & 1) * 2, nb0 = (wave & 1) * NB;
+    const int64_t grp = (b * nchunks + c) * ngroups + g;
+
+    // inputs are already summed over the head slices (slice_sum_kernel)
+    floatx16 dG[1][2], aC[1][NB], aB[1][NB];
+    acc_zero(dG);
+    {
+        const float* gp = dGp + grp * (int64_t)(kQ * kQ);
+        const float* cp = dCp + grp * (int64_t)(kQ * N);
+        const float* bp = dBp + grp * (int64_t)(kQ * N);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int row = rb * 32 + acc_row(lane, v);
+#pragma unroll
+            for (int jb = 0; jb < 2; ++jb)
+                if (cb0 + jb <= rb) dG[0][jb][v] = gp[row * kQ + (cb0 + jb) * 32 + r];
+#pragma unroll
+            for (int jn = 0; jn < NB; ++jn) {
+                aC[0][jn][v] = cp[row * N + (nb0 + jn) * 32 + r];
+                aB[0][jn][v] = bp[row * N + (nb0 + jn) * 32 + r];
+            }
+        }
+    }
     constexpr int NPASS = sizeof(T) == 2 ? 2 : 1;
-
-    // ---- F1: dC[i][n] += sum_{j<=i} dG[i][j] B[j][n]
-    stage_transposed<T, kQ, N, 512, false>(sT2, LDQ, Bp, Bsl, valid, nullptr, tid);
+    // dC[i][n] += sum_{j<=i} dG[i][j] B[j][n]
+    stage_rows<T, N, kQ, 512, false>(sT2, LDQ, Bt + grp * (int64_t)(N * kQ), kQ, N, nullptr, tid);
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
 #pragma unroll
         for (int jb = 0; jb < 2; ++jb)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int i = rb * 32 + acc_row(lane, v), j = (cb0 + jb) * 32 + acc_col(lane);
+                const int i = rb * 32 + acc_row(lane, v), j = (cb0 + jb) * 32 + r;
                 const float full = dG[0][jb][v];
                 const T hi = from_f32<T>(full);
                 sA2[i * LDQ + j] = pass == 0 ? hi : from_f32<T>(full - to_f32(hi));
             }
         __syncthreads();
-        wave_mma<1, NB>(dC, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, 0, (rb + 1) * 32);
+        wave_mma<1, NB>(aC, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, 0, (rb + 1) * 32);
         __syncthreads();
     }
-
-    // ---- F2: dB[j][n] += sum_{i>=j} dG[i][j] C[i][n]
-    stage_transposed<T, kQ, N, 512, false>(sT2, LDQ, Cp, Csl, valid, nullptr, tid);
+    // dB[j][n] += sum_{i>=j} dG[i][j] C[i][n]
+    stage_rows<T, N, kQ, 512, false>(sT2, LDQ, Ct + grp * (int64_t)(N * kQ), kQ, N, nullptr, tid);
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
 #pragma unroll
         for (int jb = 0; jb < 2; ++jb)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int i = rb * 32 + acc_row(lane, v), j = (cb0 + jb) * 32 + acc_col(lane);
+                const int i = rb * 32 + acc_row(lane, v), j = (cb0 + jb) * 32 + r;
                 const float full = dG[0][jb][v];
                 const T hi = from_f32<T>(full);
                 sA2[j * LDQ + i] = pass == 0 ? hi : from_f32<T>(full - to_f32(hi));
             }
         __syncthreads();
-        wave_mma<1, NB>(dB, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, rb * 32, kQ);
+        wave_mma<1, NB>(aB, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, rb * 32, kQ);
         __syncthreads();
     }
-
-    // ---- store partials [b][c][g][slice][Q][N]
-    const int64_t pt = (((b * nchunks + c) * ngroups + g) * nslices + slice) * (int64_t)(kQ * N);
+    T* dBo = dB + b * dBsb + t0 * dBsl + g * dBsg;
+    T* dCo = dC + b * dCsb + t0 * dCsl + g * dCsg;
 #pragma unroll
     for (int jn = 0; jn < NB; ++jn)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            const int row = rb * 32 + acc_row(lane, v), col = (nb0 + jn) * 32 + acc_col(lane);
-            dCp[pt + row * N + col] = dC[0][jn][v];
-            dBp[pt + row * N + col] = dB[0][jn][v];
+            const int row = rb * 32 + acc_row(lane, v), col = (nb0 + jn) * 32 + r;
+            if (row < valid) {
+                dCo[(int64_t)row * dCsl + col] = from_f32<T>(aC[0][jn][v]);
+                dBo[(int64_t)row * dBsl + col] = from_f32<T>(aB[0][jn][v]);
+            }
         }
-}
-
-// dB / dC = sum over head slices of the partials, cast to the activation type.  One thread per 4 state columns.
-template <typename T>
-__global__ void __launch_bounds__(256)
-bc_reduce_kernel(const float* __restrict__ dBp, const float* __restrict__ dCp, T* __restrict__ dB, T* __restrict__ dC,
-                 int64_t nb, int64_t seqlen, int64_t ngroups, int64_t nchunks, int64_t nslices, int N,
-                 int64_t dBsb, int64_t dBsl, int64_t dBsg, int64_t dCsb, int64_t dCsl, int64_t dCsg) {
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int n4s = N / 4;
-    const int64_t total = nb * seqlen * ngroups * n4s;
-    if (idx >= total) return;
-    const int n4 = (int)(idx % n4s) * 4;
-    const int64_t g = (idx / n4s) % ngroups;
-    const int64_t t = (idx / n4s / ngroups) % seqlen;
-    const int64_t b = idx / n4s / ngroups / seqlen;
-    const int64_t c = t / kQ, i = t % kQ;
-    const int64_t base = (((b * nchunks + c) * ngroups + g) * nslices) * (int64_t)(kQ * N) + i * N + n4;
-    floatx4 sb = {0.f, 0.f, 0.f, 0.f}, sc = {0.f, 0.f, 0.f, 0.f};
-    for (int64_t s = 0; s < nslices; ++s) {
-        sb += *reinterpret_cast<const floatx4*>(dBp + base + s * (int64_t)(kQ * N));
-        sc += *reinterpret_cast<const floatx4*>(dCp + base + s * (int64_t)(kQ * N));
-    }
-    T* ob = dB + b * dBsb + t * dBsl + g * dBsg + n4;
-    T* oc = dC + b * dCsb + t * dCsl + g * dCsg + n4;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) { ob[q] = from_f32<T>(sb[q]); oc[q] = from_f32<T>(sc[q]); }
 }
 
 // dA[h] = sum_{b,c} dAp[b][h][c], dD likewise.  One block per head.
@@ -455,18 +383,12 @@ __global__ void copy_f32_kernel(const float* __restrict__ src, float* __restrict
     if (i < n) dst[i] = src ? src[i] : 0.f;
 }
 
+template <typename T, int P>
+size_t dg_smem() { return (size_t)(8 * kQ + 2 * kQ + 4 * kQ) * sizeof(float) + ((size_t)2 * kQ * lds_ld<T>(P) + (dg_g_in_lds<T, P>() ? (size_t)kQ * lds_ld<T>(kQ) : 0)) * sizeof(T); }
 template <typename T, int P, int N>
-size_t dx_smem() {
-    const size_t a = (size_t)(kQ + P) * lds_ld<T>(N), b = (size_t)(kQ + P) * lds_ld<T>(kQ);
-    return (4 * kQ + 12) * sizeof(float) + (a > b ? a : b) * sizeof(T);
-}
-template <typename T, int P, int N>
-size_t gg_smem() {
-    size_t a = (size_t)2 * kQ * lds_ld<T>(P), b = (size_t)(kQ + N) * lds_ld<T>(kQ), c = (size_t)(kQ + N) * lds_ld<T>(P);
-    size_t m = a > b ? a : b;
-    m = m > c ? m : c;
-    return (14 * kQ + 4) * sizeof(float) + m * sizeof(T);
-}
+size_t off_smem(bool side_c) { return (size_t)(8 * kQ + 2 * kQ) * sizeof(float) + ((size_t)(kQ + N) * lds_ld<T>(P) + ((side_c && off_c_in_lds<T, P, N>()) ? (size_t)kQ * lds_ld<T>(N) : 0)) * sizeof(T); }
+template <typename T, int N>
+size_t bcf_smem() { return (size_t)(kQ + N) * lds_ld<T>(kQ) * sizeof(T); }
 
 template <typename T, int P, int N>
 int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
@@ -474,59 +396,93 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
     const SsdWorkspace w = ssd_carve(p, p->workspace, true);
     const int dt_f32 = p->dt_dtype == M2_F32;
     const T* x = static_cast<const T*>(p->x);
-    const T* Bm = static_cast<const T*>(p->B);
     const T* Cm = static_cast<const T*>(p->C);
     const T* dy = static_cast<const T*>(p->dy);
+    const dim3 grid_s((unsigned)nc, (unsigned)(p->ngroups * w.nslices), (unsigned)p->batch);
+    M2_REQUIRE(p->ngroups * w.nslices <= 65535, M2_ERR_SHAPE, "ssd_bwd: too many group slices");
     int rc;
-    // recompute G, S_prev, final state
+    // recompute G (+ operand tiles), S_prev, final state
     if ((rc = ssd_launch_states<T, P, N>(p, w, w.sfinal, st))) return rc;
     // local dS contributions (reuses the `local` region) and the reverse recurrence
     {
         auto k = chunk_state_kernel<T, P, N, true>;
         const size_t sm = state_smem<T, P, N>();
         if ((rc = allow_smem(k, sm))) return rc;
-        k<<<dim3((unsigned)nc, (unsigned)p->nheads, (unsigned)p->batch), 256, sm, st>>>(
-            dy, p->dt, dt_f32, p->A, Cm, w.local, nullptr, p->seqlen, p->nheads, p->ngroups, nc,
-            p->dy_stride_b, p->dy_stride_l, p->dy_stride_h, p->dt_stride_b, p->dt_stride_l,
-            p->C_stride_b, p->C_stride_l, p->C_stride_g);
+        int64_t ns, hps;
+        ssd_head_slicing(p, 1024, &ns, &hps);
+        k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * ns), (unsigned)p->batch), 256, sm, st>>>(
+            dy, p->dt, dt_f32, p->A, static_cast<const T*>(w.Ct), w.local, nullptr, p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
+            p->dy_stride_b, p->dy_stride_l, p->dy_stride_h, p->dt_stride_b, p->dt_stride_l);
         if ((rc = check_launch("ssd chunk_state_kernel<dstate>"))) return rc;
-        state_scan_kernel<T, P * N, true><<<dim3((unsigned)p->nheads, (unsigned)p->batch), 256, 0, st>>>(
+        state_scan_kernel<T, P * N, true><<<dim3((unsigned)p->nheads, (unsigned)p->batch, kScanSplit), 256, 0, st>>>(
             w.local, w.lam, p->d_final_state, static_cast<T*>(w.dprev), p->d_initial_state,
             static_cast<const T*>(w.prev), w.sfinal, w.dlam, p->nheads, nc);
         if ((rc = check_launch("ssd state_scan_kernel<reverse>"))) return rc;
     }
     {
-        auto k = group_grad_kernel<T, P, N>;
-        const size_t sm = gg_smem<T, P, N>();
+        auto k = dg_kernel<T, P>;
+        const size_t sm = dg_smem<T, P>();
         if ((rc = allow_smem(k, sm))) return rc;
-        M2_REQUIRE(p->ngroups * w.nslices <= 65535, M2_ERR_SHAPE, "ssd_bwd: too many group slices");
-        k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * w.nslices), (unsigned)p->batch), 512, sm, st>>>(
-            x, p->dt, dt_f32, p->A, Bm, Cm, dy, static_cast<const T*>(w.prev), static_cast<const T*>(w.dprev), w.G, w.dBp, w.dCp, w.dl,
-            p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice,
-            p->x_stride_b, p->x_stride_l, p->x_stride_h, p->dt_stride_b, p->dt_stride_l,
-            p->B_stride_b, p->B_stride_l, p->B_stride_g, p->C_stride_b, p->C_stride_l, p->C_stride_g,
-            p->dy_stride_b, p->dy_stride_l, p->dy_stride_h);
-        if ((rc = check_launch("ssd group_grad_kernel"))) return rc;
+        k<<<grid_s, 512, sm, st>>>(x, p->dt, dt_f32, p->A, dy, static_cast<const T*>(w.Gm), w.dGp, w.dl,
+                                   p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice,
+                                   p->x_stride_b, p->x_stride_l, p->x_stride_h, p->dt_stride_b, p->dt_stride_l,
+                                   p->dy_stride_b, p->dy_stride_l, p->dy_stride_h);
+        if ((rc = check_launch("ssd dg_kernel"))) return rc;
     }
     {
-        auto k = dx_kernel<T, P, N>;
-        const size_t sm = dx_smem<T, P, N>();
-        if ((rc = allow_smem(k, sm))) return rc;
-        k<<<dim3((unsigned)nc, (unsigned)p->nheads, (unsigned)p->batch), 256, sm, st>>>(
-            x, p->dt, dt_f32, p->A, Bm, p->D, w.G, w.dl, dy, static_cast<const T*>(w.dprev), w.dlam,
-            static_cast<T*>(p->dx), p->ddt, w.dAp, w.dDp, p->seqlen, p->nheads, p->ngroups, nc,
-            p->x_stride_b, p->x_stride_l, p->x_stride_h, p->dt_stride_b, p->dt_stride_l,
-            p->B_stride_b, p->B_stride_l, p->B_stride_g,
-            p->dy_stride_b, p->dy_stride_l, p->dy_stride_h, p->dx_stride_b, p->dx_stride_l, p->dx_stride_h,
-            p->ddt_stride_b, p->ddt_stride_l);
-        if ((rc = check_launch("ssd dx_kernel"))) return rc;
+        auto kc = off_kernel<T, P, N, true>;
+        auto kb = off_kernel<T, P, N, false>;
+        const size_t smc = off_smem<T, P, N>(true), sm = off_smem<T, P, N>(false);
+        if ((rc = allow_smem(kc, smc))) return rc;
+        if ((rc = allow_smem(kb, sm))) return rc;
+        kc<<<grid_s, 512, smc, st>>>(dy, p->dy_stride_b, p->dy_stride_l, p->dy_stride_h, p->dt, dt_f32, p->A,
+                                    static_cast<const T*>(w.prev), Cm, p->C_stride_b, p->C_stride_l, p->C_stride_g,
+                                    w.dCp, w.dlc, p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice,
+                                    p->dt_stride_b, p->dt_stride_l);
+        if ((rc = check_launch("ssd off_kernel<C>"))) return rc;
+        kb<<<grid_s, 512, sm, st>>>(x, p->x_stride_b, p->x_stride_l, p->x_stride_h, p->dt, dt_f32, p->A,
+                                    static_cast<const T*>(w.dprev), nullptr, 0, 0, 0,
+                                    w.dBp, nullptr, p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice,
+                                    p->dt_stride_b, p->dt_stride_l);
+        if ((rc = check_launch("ssd off_kernel<B>"))) return rc;
     }
     {
-        const int64_t total = p->batch * p->seqlen * p->ngroups * (N / 4);
-        bc_reduce_kernel<T><<<(unsigned)ceil_div(total, (int64_t)256), 256, 0, st>>>(
-            w.dBp, w.dCp, static_cast<T*>(p->dB), static_cast<T*>(p->dC), p->batch, p->seqlen, p->ngroups, nc, w.nslices, N,
+        DiagArgs a{};
+        a.dt = p->dt; a.dt_f32 = dt_f32; a.A = p->A; a.D = p->D;
+        a.Aoff = p->B; a.Ao_sb = p->B_stride_b; a.Ao_sl = p->B_stride_l; a.Ao_sg = p->B_stride_g;
+        a.Gd = w.Gmt; a.S = w.dprev;
+        a.Z = p->dy; a.Z_sb = p->dy_stride_b; a.Z_sl = p->dy_stride_l; a.Z_sh = p->dy_stride_h;
+        a.dt_sb = p->dt_stride_b; a.dt_sl = p->dt_stride_l;
+        a.seqlen = p->seqlen; a.nheads = p->nheads; a.ngroups = p->ngroups; a.nchunks = nc;
+        ssd_head_slicing(p, 1024, &a.nslices, &a.hps);
+        a.X = p->x; a.X_sb = p->x_stride_b; a.X_sl = p->x_stride_l; a.X_sh = p->x_stride_h;
+        a.dX = p->dx; a.dX_sb = p->dx_stride_b; a.dX_sl = p->dx_stride_l; a.dX_sh = p->dx_stride_h;
+        a.ddt = p->ddt; a.ddt_sb = p->ddt_stride_b; a.ddt_sl = p->ddt_stride_l;
+        a.dl_diag = w.dl; a.dl_c = w.dlc; a.dlam = w.dlam; a.dAp = w.dAp; a.dDp = w.dDp;
+        auto k = diag_off_kernel<T, P, N, true>;
+        const size_t sm = diag_smem<T, P, N, true>();
+        if ((rc = allow_smem(k, sm))) return rc;
+        k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * a.nslices), (unsigned)p->batch), 256, sm, st>>>(a);
+        if ((rc = check_launch("ssd diag_off_kernel<bwd>"))) return rc;
+    }
+    {
+        auto k = bc_final_kernel<T, N>;
+        const size_t sm = bcf_smem<T, N>();
+        if ((rc = allow_smem(k, sm))) return rc;
+        const int64_t ngrp = p->batch * nc * p->ngroups;
+        const float *gs = w.dGp, *cs = w.dCp, *bs = w.dBp;
+        if (w.nslices > 1) {
+            slice_sum_kernel<<<(unsigned)ceil_div(ngrp * kQ * kQ / 4, (int64_t)256), 256, 0, st>>>(w.dGp, w.dGs, ngrp, w.nslices, (int64_t)kQ * kQ);
+            slice_sum_kernel<<<(unsigned)ceil_div(ngrp * kQ * N / 4, (int64_t)256), 256, 0, st>>>(w.dCp, w.dCs, ngrp, w.nslices, (int64_t)kQ * N);
+            slice_sum_kernel<<<(unsigned)ceil_div(ngrp * kQ * N / 4, (int64_t)256), 256, 0, st>>>(w.dBp, w.dBs, ngrp, w.nslices, (int64_t)kQ * N);
+            if ((rc = check_launch("ssd slice_sum_kernel"))) return rc;
+            gs = w.dGs; cs = w.dCs; bs = w.dBs;
+        }
+        k<<<dim3((unsigned)nc, (unsigned)p->ngroups, (unsigned)p->batch), 512, sm, st>>>(
+            gs, cs, bs, static_cast<const T*>(w.Bt), static_cast<const T*>(w.Ct),
+            static_cast<T*>(p->dB), static_cast<T*>(p->dC), p->seqlen, p->ngroups, nc,
             p->dB_stride_b, p->dB_stride_l, p->dB_stride_g, p->dC_stride_b, p->dC_stride_l, p->dC_stride_g);
-        if ((rc = check_launch("ssd bc_reduce_kernel"))) return rc;
+        if ((rc = check_launch("ssd bc_final_kernel"))) return rc;
         ad_reduce_kernel<<<(unsigned)p->nheads, 256, 0, st>>>(w.dAp, w.dDp, p->dA, p->D ? p->dD : nullptr, p->batch, p->nheads, nc);
         if ((rc = check_launch("ssd ad_reduce_kernel"))) return rc;
     }

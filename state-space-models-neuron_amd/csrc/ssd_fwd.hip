@@ -121,15 +121,21 @@ int ssd_fwd_impl(const m2_ssd_params* p, hipStream_t st) {
     const SsdWorkspace w = ssd_carve(p, p->workspace, false);
     int rc;
     if ((rc = ssd_launch_states<T, P, N>(p, w, p->final_state, st))) return rc;
-    auto k = chunk_scan_kernel<T, P, N>;
-    const size_t sm = scan_smem<T, P, N>();
+    DiagArgs a{};
+    a.dt = p->dt; a.dt_f32 = p->dt_dtype == M2_F32; a.A = p->A; a.D = p->D;
+    a.Aoff = p->C; a.Ao_sb = p->C_stride_b; a.Ao_sl = p->C_stride_l; a.Ao_sg = p->C_stride_g;
+    a.Gd = w.Gm; a.S = w.prev;
+    a.Z = p->x; a.Z_sb = p->x_stride_b; a.Z_sl = p->x_stride_l; a.Z_sh = p->x_stride_h;
+    a.dt_sb = p->dt_stride_b; a.dt_sl = p->dt_stride_l;
+    a.seqlen = p->seqlen; a.nheads = p->nheads; a.ngroups = p->ngroups; a.nchunks = nc;
+    ssd_head_slicing(p, 1024, &a.nslices, &a.hps);
+    a.Y = p->y; a.Y_sb = p->y_stride_b; a.Y_sl = p->y_stride_l; a.Y_sh = p->y_stride_h;
+    auto k = diag_off_kernel<T, P, N, false>;
+    const size_t sm = diag_smem<T, P, N, false>();
     if ((rc = allow_smem(k, sm))) return rc;
-    k<<<dim3((unsigned)nc, (unsigned)p->nheads, (unsigned)p->batch), 256, sm, st>>>(
-        static_cast<const T*>(p->x), p->dt, p->dt_dtype == M2_F32, p->A, static_cast<const T*>(p->C), p->D, w.G,
-        static_cast<const T*>(w.prev), static_cast<T*>(p->y), p->seqlen, p->nheads, p->ngroups, nc,
-        p->x_stride_b, p->x_stride_l, p->x_stride_h, p->dt_stride_b, p->dt_stride_l,
-        p->C_stride_b, p->C_stride_l, p->C_stride_g, p->y_stride_b, p->y_stride_l, p->y_stride_h);
-    return check_launch("ssd chunk_scan_kernel");
+    M2_REQUIRE(p->ngroups * a.nslices <= 65535, M2_ERR_SHAPE, "ssd_fwd: too many group slices");
+    k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * a.nslices), (unsigned)p->batch), 256, sm, st>>>(a);
+    return check_launch("ssd diag_off_kernel<fwd>");
 }
 
 }  // namespace

@@ -1,6 +1,7 @@
 // Host-side helpers shared by the SSD forward and backward launchers.
 #pragma once
 #include "ssd_kernels.hpp"
+#include "ssd_diag.hpp"
 
 namespace m2 {
 
@@ -11,8 +12,10 @@ namespace m2 {
 // per-(b,chunk,group,head-slice) fp32 partials of dB and dC.
 struct SsdWorkspace {
     float* G = nullptr; float* local = nullptr; void* prev = nullptr; float* lam = nullptr;
+    void* Gm = nullptr; void* Gmt = nullptr; void* Bt = nullptr; void* Ct = nullptr;
     float* sfinal = nullptr; void* dprev = nullptr; float* dlam = nullptr;
-    float* dAp = nullptr; float* dDp = nullptr; float* dBp = nullptr; float* dCp = nullptr; float* dl = nullptr;
+    float* dAp = nullptr; float* dDp = nullptr; float* dBp = nullptr; float* dCp = nullptr; float* dl = nullptr; float* dlc = nullptr; float* dGp = nullptr;
+    float* dGs = nullptr; float* dBs = nullptr; float* dCs = nullptr;   // partials summed over the head slices
     int64_t nslices = 1, heads_per_slice = 1;
     size_t bytes = 0;
 };
@@ -34,6 +37,22 @@ inline void ssd_bwd_slicing(const m2_ssd_params* p, int64_t* nslices, int64_t* h
     *hps = hpg / best;
 }
 
+// Forward / dx kernels: a workgroup loops over `hps` heads of one group (operand fragments shared by the group stay
+// in registers); choose the slice count so that the grid has at least ~1024 workgroups when the shape allows.
+inline void ssd_head_slicing(const m2_ssd_params* p, int64_t target, int64_t* nslices, int64_t* hps) {
+    const int64_t nc = ceil_div(p->seqlen, (int64_t)kQ);
+    const int64_t hpg = p->nheads / p->ngroups;
+    const int64_t base = p->batch * nc * p->ngroups;
+    int64_t best = 1;
+    for (int64_t s = 1; s <= hpg; ++s) {
+        if (hpg % s) continue;
+        best = s;
+        if (base * s >= target) break;
+    }
+    *nslices = best;
+    *hps = hpg / best;
+}
+
 inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd) {
     const int64_t nc = ceil_div(p->seqlen, (int64_t)kQ);
     const size_t esz = p->dtype == M2_F32 ? 4 : 2;
@@ -47,17 +66,27 @@ inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd) {
     w.local = reinterpret_cast<float*>(take(tiles * 4));
     w.prev = take(tiles * esz);
     w.lam = reinterpret_cast<float*>(take(bhc * 4));
+    const size_t grp = (size_t)p->batch * nc * p->ngroups;
+    w.Gm = take(grp * kQ * kQ * esz);
+    w.Gmt = take(grp * kQ * kQ * esz);
+    w.Bt = take(grp * p->dstate * kQ * esz);
+    w.Ct = take(grp * p->dstate * kQ * esz);
     if (bwd) {
         ssd_bwd_slicing(p, &w.nslices, &w.heads_per_slice);
         w.sfinal = reinterpret_cast<float*>(take((size_t)p->batch * p->nheads * p->headdim * p->dstate * 4));
         w.dprev = take(tiles * esz);
-        w.dlam = reinterpret_cast<float*>(take(bhc * 4));
+        w.dlam = reinterpret_cast<float*>(take(bhc * 4 * kScanSplit));
         w.dAp = reinterpret_cast<float*>(take(bhc * 4));
         w.dDp = reinterpret_cast<float*>(take(bhc * 4));
         w.dl = reinterpret_cast<float*>(take(bhc * kQ * 4));
+        w.dlc = reinterpret_cast<float*>(take(bhc * kQ * 4));
+        w.dGp = reinterpret_cast<float*>(take((size_t)p->batch * nc * p->ngroups * w.nslices * kQ * kQ * 4));
         const size_t part = (size_t)p->batch * nc * p->ngroups * w.nslices * kQ * p->dstate * 4;
         w.dBp = reinterpret_cast<float*>(take(part));
         w.dCp = reinterpret_cast<float*>(take(part));
+        w.dGs = reinterpret_cast<float*>(take((size_t)p->batch * nc * p->ngroups * kQ * kQ * 4));
+        w.dBs = reinterpret_cast<float*>(take((size_t)p->batch * nc * p->ngroups * kQ * p->dstate * 4));
+        w.dCs = reinterpret_cast<float*>(take((size_t)p->batch * nc * p->ngroups * kQ * p->dstate * 4));
     }
     w.bytes = off + 256;
     return w;
@@ -94,7 +123,7 @@ inline int allow_smem(K kernel, size_t bytes) {
 }
 
 template <typename T, int P, int N>
-inline size_t state_smem() { return (3 * kQ + 4) * sizeof(float) + (size_t)(P + N) * lds_ld<T>(kQ) * sizeof(T); }
+inline size_t state_smem() { return (size_t)(P + N) * lds_ld<T>(kQ) * sizeof(T); }
 template <typename T>
 inline size_t cb_smem() { return (size_t)2 * kQ * lds_ld<T>(64) * sizeof(T); }
 
@@ -112,7 +141,7 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
         const size_t sm = cb_smem<T>();
         if ((rc = allow_smem(k, sm))) return rc;
         k<<<dim3((unsigned)nc, (unsigned)p->ngroups, (unsigned)p->batch), 256, sm, st>>>(
-            Bm, Cm, w.G, p->seqlen, p->ngroups, nc, p->B_stride_b, p->B_stride_l, p->B_stride_g,
+            Bm, Cm, w.G, static_cast<T*>(w.Gm), static_cast<T*>(w.Gmt), static_cast<T*>(w.Bt), static_cast<T*>(w.Ct), p->seqlen, p->ngroups, nc, p->B_stride_b, p->B_stride_l, p->B_stride_g,
             p->C_stride_b, p->C_stride_l, p->C_stride_g);
         if ((rc = check_launch("ssd cb_kernel"))) return rc;
     }
@@ -120,14 +149,16 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
         auto k = chunk_state_kernel<T, P, N, false>;
         const size_t sm = state_smem<T, P, N>();
         if ((rc = allow_smem(k, sm))) return rc;
-        k<<<dim3((unsigned)nc, (unsigned)p->nheads, (unsigned)p->batch), 256, sm, st>>>(
-            x, p->dt, dt_f32, p->A, Bm, w.local, w.lam, p->seqlen, p->nheads, p->ngroups, nc,
-            p->x_stride_b, p->x_stride_l, p->x_stride_h, p->dt_stride_b, p->dt_stride_l,
-            p->B_stride_b, p->B_stride_l, p->B_stride_g);
+        int64_t ns, hps;
+        ssd_head_slicing(p, 1024, &ns, &hps);
+        M2_REQUIRE(p->ngroups * ns <= 65535, M2_ERR_SHAPE, "ssd: too many group slices");
+        k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * ns), (unsigned)p->batch), 256, sm, st>>>(
+            x, p->dt, dt_f32, p->A, static_cast<const T*>(w.Bt), w.local, w.lam, p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
+            p->x_stride_b, p->x_stride_l, p->x_stride_h, p->dt_stride_b, p->dt_stride_l);
         if ((rc = check_launch("ssd chunk_state_kernel"))) return rc;
     }
     {
-        state_scan_kernel<T, P * N, false><<<dim3((unsigned)p->nheads, (unsigned)p->batch), 256, 0, st>>>(
+        state_scan_kernel<T, P * N, false><<<dim3((unsigned)p->nheads, (unsigned)p->batch, kScanSplit), 256, 0, st>>>(
             w.local, w.lam, p->initial_state, static_cast<T*>(w.prev), final_out, nullptr, nullptr, nullptr, p->nheads, nc);
         if ((rc = check_launch("ssd state_scan_kernel"))) return rc;
     }

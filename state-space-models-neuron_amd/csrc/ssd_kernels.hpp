@@ -28,16 +28,22 @@ struct SsdDims {
 };
 
 // ------------------------------------------------------------------------------------------
-// G[b][c][g][i][j] = sum_n C[i][n] * B[j][n].   grid (nchunks, ngroups, batch), 256 threads.
-// Only 32x32 blocks with block-row >= block-col are consumed (causal); the upper-right
-// 64x64 quadrant is neither computed nor written.
+// Per (batch, chunk, group): G = C B^T and the head-independent operand tiles every other kernel reuses.
+//   Gf  [kQ][kQ] fp32            G[i][j] (all blocks with block-row >= block-col)
+//   Gm  [kQ][kQ] T               causal G:  G[i][j] for i >= j, else 0         (forward diagonal term, rows i)
+//   Gmt [kQ][kQ] T               its transpose: Gmt[j][i] = G[i][j] for i >= j (backward dx term, rows j)
+//   Bt, Ct [N][kQ] T             B and C transposed (tokens contiguous): MFMA operands of the chunk-state products
+// grid (nchunks, ngroups, batch), 256 threads.  The upper-right 64x64 quadrant of G is never consumed and is
+// neither computed nor written.
 template <typename T, int N>
 __global__ void __launch_bounds__(256)
-cb_kernel(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict__ G,
+cb_kernel(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict__ Gf, T* __restrict__ Gm, T* __restrict__ Gmt,
+          T* __restrict__ Bt, T* __restrict__ Ct,
           int64_t seqlen, int64_t ngroups, int64_t nchunks,
           int64_t Bsb, int64_t Bsl, int64_t Bsg, int64_t Csb, int64_t Csl, int64_t Csg) {
     constexpr int KB = 64;
     constexpr int LD = lds_ld<T>(KB);
+    constexpr int V = VecTraits<T>::kVec;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* sC = reinterpret_cast<T*>(smem_raw);
     T* sB = sC + kQ * LD;
@@ -47,6 +53,9 @@ cb_kernel(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict_
     const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
     const T* Bp = Bm + b * Bsb + t0 * Bsl + g * Bsg;
     const T* Cp = Cm + b * Csb + t0 * Csl + g * Csg;
+    const int64_t grp = (b * nchunks + c) * ngroups + g;
+    T* Btp = Bt + grp * (int64_t)(N * kQ);
+    T* Ctp = Ct + grp * (int64_t)(N * kQ);
     const int wm = wave >> 1, wn = wave & 1;
     floatx16 acc[2][2];
     acc_zero(acc);
@@ -55,103 +64,154 @@ cb_kernel(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict_
         stage_rows<T, kQ, KB, 256, false>(sB, LD, Bp + k0, Bsl, valid, nullptr, tid);
         __syncthreads();
         if (!(wm == 0 && wn == 1)) wave_mma<2, 2>(acc, sC + wm * 64 * LD, LD, sB + wn * 64 * LD, LD, 0, KB);
+        // transposed copies of this 64-column slab: thread -> (state column n, group of V tokens)
+        for (int e = tid; e < KB * (kQ / V); e += 256) {
+            const int n = e % KB, s0 = (e / KB) * V;
+            T vb[V], vc[V];
+#pragma unroll
+            for (int q = 0; q < V; ++q) { vb[q] = sB[(s0 + q) * LD + n]; vc[q] = sC[(s0 + q) * LD + n]; }
+            *reinterpret_cast<uint4*>(Btp + (int64_t)(k0 + n) * kQ + s0) = *reinterpret_cast<const uint4*>(vb);
+            *reinterpret_cast<uint4*>(Ctp + (int64_t)(k0 + n) * kQ + s0) = *reinterpret_cast<const uint4*>(vc);
+        }
         __syncthreads();
     }
     if (wm == 0 && wn == 1) return;
-    float* Gp = G + ((b * nchunks + c) * ngroups + g) * (int64_t)(kQ * kQ);
+    float* Gfp = Gf + grp * (int64_t)(kQ * kQ);
+    T* Gmp = Gm + grp * (int64_t)(kQ * kQ);
+    T* Gmtp = Gmt + grp * (int64_t)(kQ * kQ);
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < 2; ++j) {
+            if (wm * 2 + i < wn * 2 + j) continue;          // block above the diagonal
+            const int col = wn * 64 + j * 32 + acc_col(lane);
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = wm * 64 + i * 32 + acc_row(lane, v);
-                const int col = wn * 64 + j * 32 + acc_col(lane);
-                Gp[row * kQ + col] = acc[i][j][v];
+            for (int q = 0; q < 4; ++q) {
+                const int rowq = wm * 64 + i * 32 + 8 * q + 4 * (lane >> 5);
+                T mt[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int row = rowq + e;
+                    const float gv = acc[i][j][4 * q + e];
+                    const float gm = row >= col ? gv : 0.f;
+                    Gfp[row * kQ + col] = gv;
+                    Gmp[row * kQ + col] = from_f32<T>(gm);
+                    mt[e] = from_f32<T>(gm);
+                }
+                *reinterpret_cast<RawVec<T, 4>*>(Gmtp + col * kQ + rowq) = *reinterpret_cast<const RawVec<T, 4>*>(mt);
             }
+        }
 }
 
 // ------------------------------------------------------------------------------------------
-// Local chunk state.  grid (nchunks, nheads, batch), 256 threads.
+// Local chunk state.  grid (nchunks, ngroups * nslices, batch), 256 threads; a workgroup loops over `hps` heads.
 //   DSTATE == false:  out[p][n] = sum_j (dt_j e^{Lam-l_j}) x[j][p] * B[j][n]      (forward)
 //   DSTATE == true :  out[p][n] = sum_i e^{l_i} dy[i][p] * C[i][n]                (backward)
-// Also writes lam[b][h][c] = Lam.  `X` is x or dy, `M` is B or C.
+// `X` is x or dy; `Mt` is the group's B or C tile already transposed to [N][kQ] (tokens contiguous) by cb_kernel,
+// staged into LDS once per workgroup.  Per head only the x tile moves: it is loaded 16 bytes at a time, scaled in
+// fp32 and written transposed; the next head's tile is prefetched into registers while the MFMAs run.
+// Also writes lam[b][h][c] = Lam.
 template <typename T, int P, int N, bool DSTATE>
 __global__ void __launch_bounds__(256)
 chunk_state_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f32, const float* __restrict__ A,
-                   const T* __restrict__ M, float* __restrict__ out, float* __restrict__ lam,
-                   int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks,
-                   int64_t Xsb, int64_t Xsl, int64_t Xsh, int64_t dtsb, int64_t dtsl,
-                   int64_t Msb, int64_t Msl, int64_t Msg) {
+                   const T* __restrict__ Mt, float* __restrict__ out, float* __restrict__ lam,
+                   int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks, int64_t nslices, int64_t hps,
+                   int64_t Xsb, int64_t Xsl, int64_t Xsh, int64_t dtsb, int64_t dtsl) {
     constexpr int LD = lds_ld<T>(kQ);
+    constexpr int V = VecTraits<T>::kVec;
+    constexpr int NIT = (P / V) / 2;              // 16-byte vectors per thread per head (thread <-> fixed token)
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    float* s_l = reinterpret_cast<float*>(smem_raw);
-    float* s_dt = s_l + kQ;
-    float* s_sc = s_dt + kQ;
-    float* s_tmp = s_sc + kQ;          // 4 floats
-    T* sX = reinterpret_cast<T*>(s_tmp + 4);   // [P][LD]
-    T* sM = sX + P * LD;                       // [N][LD]
+    T* sX = reinterpret_cast<T*>(smem_raw);        // [P][LD]   x^T scaled
+    T* sM = sX + P * LD;                           // [N][LD]   B^T or C^T
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int64_t c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    const int64_t g = h / (nheads / ngroups);
+    const int64_t c = blockIdx.x, b = blockIdx.z;
+    const int64_t g = blockIdx.y / nslices, slice = blockIdx.y % nslices;
+    const int64_t hpg = nheads / ngroups;
     const int64_t t0 = c * kQ;
     const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
+    const int tok = tid & (kQ - 1), cvh = tid >> 7;       // this thread's token and channel-vector parity
 
-    chunk_cumsum_any<T>(dt, dt_f32, b * dtsb + t0 * dtsl + h, dtsl, valid, A[h], s_l, s_dt, s_tmp, tid);
-    const float Lam = s_l[kQ - 1];
-    if (tid < kQ) s_sc[tid] = DSTATE ? __expf(s_l[tid]) : s_dt[tid] * __expf(Lam - s_l[tid]);
-    __syncthreads();
-
-    stage_transposed<T, kQ, P, 256, true>(sX, LD, X + b * Xsb + t0 * Xsl + h * Xsh, Xsl, valid, s_sc, tid);
-    stage_transposed<T, kQ, N, 256, false>(sM, LD, M + b * Msb + t0 * Msl + g * Msg, Msl, valid, nullptr, tid);
-    __syncthreads();
+    stage_rows<T, N, kQ, 256, false>(sM, LD, Mt + ((b * nchunks + c) * ngroups + g) * (int64_t)(N * kQ), kQ, N, nullptr, tid);
 
     constexpr int BM = P / 64, BN = N / 64;
     const int wm = wave >> 1, wn = wave & 1;
-    floatx16 acc[BM][BN];
-    acc_zero(acc);
-    wave_mma<BM, BN>(acc, sX + wm * (P / 2) * LD, LD, sM + wn * (N / 2) * LD, LD, 0, kQ);
+    uint4 pre[NIT];
+    auto prefetch = [&](int64_t h) {
+        const T* xp = X + b * Xsb + (t0 + tok) * Xsl + h * Xsh;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it)
+            pre[it] = tok < valid ? *reinterpret_cast<const uint4*>(xp + (it * 2 + cvh) * V) : uint4{0u, 0u, 0u, 0u};
+    };
+    prefetch(g * hpg + slice * hps);
 
-    float* op = out + ((b * nchunks + c) * nheads + h) * (int64_t)(P * N);
+    for (int64_t hh = 0; hh < hps; ++hh) {
+        const int64_t h = g * hpg + slice * hps + hh;
+        float l0, l1, d0, d1;
+        wave_chunk_cumsum<T>(dt, dt_f32, b * dtsb + t0 * dtsl + h, dtsl, valid, A[h], l0, l1, d0, d1);
+        const float Lam = __shfl(l1, 63, 64);
+        // scale of this thread's token (token = lane + 64 * (wave & 1))
+        const float lt = (wave & 1) ? l1 : l0, dtt = (wave & 1) ? d1 : d0;
+        const float sc = DSTATE ? __expf(lt) : dtt * __expf(Lam - lt);
+        __syncthreads();                     // previous head's MFMAs are done with sX
 #pragma unroll
-    for (int i = 0; i < BM; ++i)
+        for (int it = 0; it < NIT; ++it) {
+            const T* el = reinterpret_cast<const T*>(&pre[it]);
 #pragma unroll
-        for (int j = 0; j < BN; ++j)
+            for (int i = 0; i < V; ++i) sX[((it * 2 + cvh) * V + i) * LD + tok] = from_f32<T>(to_f32(el[i]) * sc);
+        }
+        __syncthreads();
+        if (hh + 1 < hps) prefetch(h + 1);
+
+        floatx16 acc[BM][BN];
+        acc_zero(acc);
+        wave_mma<BM, BN>(acc, sX + wm * (P / 2) * LD, LD, sM + wn * (N / 2) * LD, LD, 0, kQ);
+        float* op = out + ((b * nchunks + c) * nheads + h) * (int64_t)(P * N);
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = wm * (P / 2) + i * 32 + acc_row(lane, v);
-                const int col = wn * (N / 2) + j * 32 + acc_col(lane);
-                op[row * N + col] = acc[i][j][v];
-            }
-    if (tid == 0 && lam) lam[(b * nheads + h) * nchunks + c] = Lam;
+        for (int i = 0; i < BM; ++i)
+#pragma unroll
+            for (int j = 0; j < BN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = wm * (P / 2) + i * 32 + acc_row(lane, v);
+                    const int col = wn * (N / 2) + j * 32 + acc_col(lane);
+                    op[row * N + col] = acc[i][j][v];
+                }
+        if (tid == 0 && lam) lam[(b * nheads + h) * nchunks + c] = Lam;
+    }
 }
 
 // ------------------------------------------------------------------------------------------
-// Inter-chunk recurrence.  grid (nheads, batch), 256 threads; each thread owns EPT float4
-// slices of the [p][n] state and walks the chunks with the running state in registers (fp32).
+// Inter-chunk recurrence.  grid (nheads, batch, kScanSplit), 256 threads; a workgroup owns 1/kScanSplit of the
+// [p][n] state of one (batch, head), each thread EPT float4 slices of it, and walks the chunks with the running
+// state in registers (fp32).  The split only exists to put enough waves on the GPU to hide memory latency.
 //
 // forward (REVERSE == false):
 //     run = init;  for c = 0..nc-1:  prev[c] = T(run);  run = e^{lam_c} run + local[c];  final = run
 // reverse (REVERSE == true), the gradient recurrence:
 //     run = dfinal;  for c = nc-1..0:  prev[c] = T(run)   (= dL/dS_new(c));
-//                                      dlam[c] = <run, S_new(c)>;   run = e^{lam_c} run + local[c]
+//                                      dlam[c][split] = <run, S_new(c)> over this workgroup's part;
+//                                      run = e^{lam_c} run + local[c]
 //     dinit = run.     S_new(c) = sprev[c+1] for c < nc-1, the fp32 final state for c = nc-1.
+constexpr int kScanSplit = 4;
+
 template <typename T, int PN, bool REVERSE>
 __global__ void __launch_bounds__(256)
 state_scan_kernel(const float* __restrict__ local, const float* __restrict__ lam, const float* __restrict__ init,
                   T* __restrict__ prev, float* __restrict__ final_out,
                   const T* __restrict__ sprev, const float* __restrict__ sfinal, float* __restrict__ dlam,
                   int64_t nheads, int64_t nchunks) {
-    constexpr int EPT = PN / 4 / 256;
-    static_assert(PN % 1024 == 0, "state size must be a multiple of 1024 elements");
-    __shared__ float red[4];
+    constexpr int EPT = PN / 4 / 256 / kScanSplit;
+    static_assert(PN % (1024 * kScanSplit) == 0, "state size must be a multiple of 4096 elements");
+    const int part0 = blockIdx.z * (PN / kScanSplit);      // first element of this workgroup's part
+    constexpr int kRedBatch = 64;
+    __shared__ float red[kRedBatch * 4];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int64_t h = blockIdx.x, b = blockIdx.y;
     const int64_t bh = b * nheads + h;
     floatx4 run[EPT];
 #pragma unroll
     for (int e = 0; e < EPT; ++e) {
-        if (init) run[e] = *reinterpret_cast<const floatx4*>(init + bh * PN + (e * 256 + tid) * 4);
+        if (init) run[e] = *reinterpret_cast<const floatx4*>(init + bh * PN + part0 + (e * 256 + tid) * 4);
         else run[e] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
 #pragma unroll 1
@@ -162,7 +222,7 @@ state_scan_kernel(const float* __restrict__ local, const float* __restrict__ lam
         float dot = 0.f;
 #pragma unroll
         for (int e = 0; e < EPT; ++e) {
-            const int off = (e * 256 + tid) * 4;
+            const int off = part0 + (e * 256 + tid) * 4;
             const floatx4 loc = *reinterpret_cast<const floatx4*>(local + tile + off);
             // store the state entering (forward) / the gradient leaving (reverse) this chunk
             T o[4];
@@ -191,17 +251,25 @@ state_scan_kernel(const float* __restrict__ local, const float* __restrict__ lam
             for (int q = 0; q < 4; ++q) run[e][q] = dec * run[e][q] + loc[q];
         }
         if (REVERSE) {
+            // per-wave partial of <dS, S_new>; the four partials are combined once per kRedBatch chunks so the
+            // streaming loop has no barrier
             dot = warp_sum(dot);
-            __syncthreads();               // red[] free again
-            if (lane == 0) red[wave] = dot;
-            __syncthreads();
-            if (tid == 0) dlam[bh * nchunks + c] = red[0] + red[1] + red[2] + red[3];
+            if (lane == 0) red[(cc % kRedBatch) * 4 + wave] = dot;
+            if ((cc % kRedBatch) == kRedBatch - 1 || cc == nchunks - 1) {
+                __syncthreads();
+                const int64_t first = cc - (cc % kRedBatch);
+                if (tid <= cc - first) {
+                    const int64_t c2 = REVERSE ? nchunks - 1 - (first + tid) : first + tid;
+                    dlam[(bh * nchunks + c2) * kScanSplit + blockIdx.z] = red[tid * 4] + red[tid * 4 + 1] + red[tid * 4 + 2] + red[tid * 4 + 3];
+                }
+                __syncthreads();
+            }
         }
     }
     if (final_out) {
 #pragma unroll
         for (int e = 0; e < EPT; ++e)
-            *reinterpret_cast<floatx4*>(final_out + bh * PN + (e * 256 + tid) * 4) = run[e];
+            *reinterpret_cast<floatx4*>(final_out + bh * PN + part0 + (e * 256 + tid) * 4) = run[e];
     }
 }
 
