@@ -87,16 +87,18 @@ diag_off_kernel(const DiagArgs a) {
     float* wv = wt_all + (wave * 4 + 2) * kQ;
     float* wu = wt_all + (wave * 4 + 3) * kQ;
 
-    // ---- head-independent A-operand fragments of the masked CB^T tile, kept in registers
-    Frag<T> fd[8];
+    // ---- head-independent A-operand fragments of the masked CB^T tile: kept in registers in the forward; the
+    //      backward (more live state) re-reads them from global memory (L2-resident) for each head
+    constexpr bool FD_RES = !BWD;
+    Frag<T> fd[FD_RES ? 8 : 1];
+    const T* Gp = static_cast<const T*>(a.Gd) + ((b * a.nchunks + c) * a.ngroups + g) * (int64_t)(kQ * kQ) + (row0 + r) * kQ;
     const T* Ao = static_cast<const T*>(a.Aoff) + b * a.Ao_sb + (t0 + row0 + r) * a.Ao_sl + g * a.Ao_sg;
     const bool ao_ok = row0 + r < valid;
-    {
-        const T* Gp = static_cast<const T*>(a.Gd) + ((b * a.nchunks + c) * a.ngroups + g) * (int64_t)(kQ * kQ) + (row0 + r) * kQ;
+    if (FD_RES) {
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             const bool used = BWD ? (ks >= 2 * wave) : (ks <= 2 * wave + 1);
-            if (used) fd[ks] = load_frag(Gp + ks * 16 + kh8);
+            if (used) fd[FD_RES ? ks : 0] = load_frag(Gp + ks * 16 + kh8);
         }
     }
 
@@ -233,7 +235,7 @@ diag_off_kernel(const DiagArgs a) {
                     else f[e] = (k >= jrow) ? __expf(wl[k] - l_row) : 0.f;
                 }
             }
-            const Frag<T> af = scale_frag(fd[ks], f);
+            const Frag<T> af = scale_frag(FD_RES ? fd[FD_RES ? ks : 0] : load_frag(Gp + ks * 16 + kh8), f);
 #pragma unroll
             for (int j = 0; j < BN; ++j) {
                 const Frag<T> bf = load_frag(sZt + (j * 32 + r) * LDQ + ks * 16 + kh8);

@@ -22,7 +22,7 @@ struct SsdWorkspace {
 
 // Heads of one group are processed by a workgroup in slices of `heads_per_slice`, so that the
 // group-level dB/dC reductions happen in registers; slices are chosen to give the GPU
-// at least ~768 workgroups when the shape allows.
+// at least 512 workgroups (two per CU) when the shape allows.
 inline void ssd_bwd_slicing(const m2_ssd_params* p, int64_t* nslices, int64_t* hps) {
     const int64_t nc = ceil_div(p->seqlen, (int64_t)kQ);
     const int64_t hpg = p->nheads / p->ngroups;
@@ -31,7 +31,7 @@ inline void ssd_bwd_slicing(const m2_ssd_params* p, int64_t* nslices, int64_t* h
     for (int64_t s = 1; s <= hpg; ++s) {
         if (hpg % s) continue;
         best = s;
-        if (base * s >= 768) break;
+        if (base * s >= 512) break;
     }
     *nslices = best;
     *hps = hpg / best;
