@@ -80,6 +80,25 @@ dg_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f32, cons
     floatx16 dG[1][2];
     acc_zero(dG);
 
+    // the next head's dY and X tiles travel global -> registers while the current head is computed
+    constexpr int V = VecTraits<T>::kVec;
+    constexpr int VPR = P / V;                     // 16-byte vectors per token row
+    constexpr int NV = kQ * VPR / 512;             // vectors per thread per tile
+    static_assert((kQ * VPR) % 512 == 0, "tile does not divide over the workgroup");
+    uint4 pdy[NV], pxx[NV];
+    auto prefetch = [&](int64_t h) {
+        const T* gy = dY + b * dYsb + t0 * dYsl + h * dYsh;
+        const T* gx = X + b * Xsb + t0 * Xsl + h * Xsh;
+#pragma unroll
+        for (int it = 0; it < NV; ++it) {
+            const int e = it * 512 + tid, rr = e / VPR, cv = e % VPR;
+            const bool ok = rr < valid;
+            pdy[it] = ok ? *reinterpret_cast<const uint4*>(gy + (int64_t)rr * dYsl + cv * V) : uint4{0u, 0u, 0u, 0u};
+            pxx[it] = ok ? *reinterpret_cast<const uint4*>(gx + (int64_t)rr * Xsl + cv * V) : uint4{0u, 0u, 0u, 0u};
+        }
+    };
+    prefetch(g * hpg + slice * hps);
+
     for (int64_t hh = 0; hh < hps; ++hh) {
         const int64_t h = g * hpg + slice * hps + hh;
         float l0, l1, d0, d1;
@@ -99,9 +118,14 @@ dg_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f32, cons
         }
 
         __syncthreads();      // previous head: tiles consumed, s_rs / s_cs consumed
-        stage_rows<T, kQ, P, 512, false>(sA, LDP, dY + b * dYsb + t0 * dYsl + h * dYsh, dYsl, valid, nullptr, tid);
-        stage_rows<T, kQ, P, 512, false>(sT, LDP, X + b * Xsb + t0 * Xsl + h * Xsh, Xsl, valid, nullptr, tid);
+#pragma unroll
+        for (int it = 0; it < NV; ++it) {
+            const int e = it * 512 + tid, rr = e / VPR, cv = e % VPR;
+            *reinterpret_cast<uint4*>(sA + rr * LDP + cv * V) = pdy[it];
+            *reinterpret_cast<uint4*>(sT + rr * LDP + cv * V) = pxx[it];
+        }
         __syncthreads();
+        if (hh + 1 < hps) prefetch(h + 1);
 
         float rsum[16], csum[2] = {0.f, 0.f};
 #pragma unroll
@@ -199,6 +223,30 @@ off_kernel(const T* __restrict__ Arow, int64_t Asb, int64_t Asl, int64_t Ash,   
     floatx16 acc[1][NB];
     acc_zero(acc);
 
+    // the next head's row tile and state tile travel global -> registers while the current head is computed
+    constexpr int V = VecTraits<T>::kVec;
+    constexpr int VPR = P / V, NVA = kQ * VPR / 512;      // row tile: vectors per token row / per thread
+    constexpr int VPS = N / V, NVS = P * VPS / 512;       // state tile [P][N]: vectors per row / per thread
+    static_assert((kQ * VPR) % 512 == 0 && (P * VPS) % 512 == 0, "tile does not divide over the workgroup");
+    uint4 pa[NVA], ps[NVS];
+    auto prefetch = [&](int64_t h) {
+        const T* ga = Arow + b * Asb + t0 * Asl + h * Ash;
+#pragma unroll
+        for (int it = 0; it < NVA; ++it) {
+            const int e = it * 512 + tid, rr = e / VPR, cv = e % VPR;
+            pa[it] = rr < valid ? *reinterpret_cast<const uint4*>(ga + (int64_t)rr * Asl + cv * V) : uint4{0u, 0u, 0u, 0u};
+        }
+        const T* gs = St + ((b * nchunks + c) * nheads + h) * (int64_t)(P * N);
+#pragma unroll
+        for (int it = 0; it < NVS; ++it) {
+            // consecutive threads take consecutive state rows p of the same 16-byte column vector (see stage_transposed)
+            const int e = it * 512 + tid, cv = e / P, pr = e % P;
+            ps[it] = *reinterpret_cast<const uint4*>(gs + (int64_t)pr * N + cv * V);
+        }
+    };
+    constexpr bool PREFETCH = SIDE_C;
+    if (PREFETCH) prefetch(g * hpg + slice * hps);
+
     for (int64_t hh = 0; hh < hps; ++hh) {
         const int64_t h = g * hpg + slice * hps + hh;
         float l0, l1, d0, d1;
@@ -208,11 +256,22 @@ off_kernel(const T* __restrict__ Arow, int64_t Asb, int64_t Asl, int64_t Ash,   
             const float Lam = __shfl(l1, 63, 64);
             ws[lane] = d0 * __expf(Lam - l0); ws[lane + 64] = d1 * __expf(Lam - l1);
         }
-        const int64_t tile = ((b * nchunks + c) * nheads + h) * (int64_t)(P * N);
         __syncthreads();
-        stage_rows<T, kQ, P, 512, false>(sA, LDP, Arow + b * Asb + t0 * Asl + h * Ash, Asl, valid, nullptr, tid);
-        stage_transposed<T, P, N, 512, false>(sT, LDP, St + tile, N, P, nullptr, tid);
+        if (!PREFETCH) prefetch(h);
+#pragma unroll
+        for (int it = 0; it < NVA; ++it) {
+            const int e = it * 512 + tid, rr = e / VPR, cv = e % VPR;
+            *reinterpret_cast<uint4*>(sA + rr * LDP + cv * V) = pa[it];
+        }
+#pragma unroll
+        for (int it = 0; it < NVS; ++it) {
+            const int e = it * 512 + tid, cv = e / P, pr = e % P;
+            const T* el = reinterpret_cast<const T*>(&ps[it]);
+#pragma unroll
+            for (int i = 0; i < V; ++i) sT[(cv * V + i) * LDP + pr] = el[i];
+        }
         __syncthreads();
+        if (PREFETCH && hh + 1 < hps) prefetch(h + 1);
         float rcv[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) rcv[v] = 0.f;
