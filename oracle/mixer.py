@@ -39,18 +39,24 @@ def rmsnorm_gated_ref(x, z, weight, n_groups=1, eps=1e-5):
 
 
 def fused_core_ref(zxBCdt, A, D, conv_w, conv_b, dt_bias, norm_w, n_groups, d_state, d_inner, d_head,
-                   chunk=128, eps=1e-5):
+                   chunk=128, eps=1e-5, handover=None):
     """zxBCdt (b, l, 2*d_inner + 2*g*n + h) -> norm_out (b, l, d_inner).
     Split order [z | xBC | dt] (``mamba2_mixer.py:265``), xBC order [x | B | C]
-    (``mamba2_kernel.py:109-115,151``)."""
+    (``mamba2_kernel.py:109-115,151``).
+
+    ``handover`` (optional callable) is applied to every tensor one stage stores for the next
+    (conv output, scan output, norm output); tests pass a round-to-bfloat16 to model what storing
+    those tensors in the activation dtype, as the reference does, costs in accuracy."""
+    if handover is None:
+        handover = lambda t: t
     b, l, _ = zxBCdt.shape
     h = d_inner // d_head
     d_conv = d_inner + 2 * n_groups * d_state
     z, xBC, dt = torch.split(zxBCdt, [d_inner, d_conv, h], dim=-1)
-    xBC = conv1d_ref(xBC, conv_w, conv_b, "silu", channels_last=True)
+    xBC = handover(conv1d_ref(xBC, conv_w, conv_b, "silu", channels_last=True))
     dt = softplus_ref(dt + dt_bias)
     x, Bm, Cm = torch.split(xBC, [d_inner, n_groups * d_state, n_groups * d_state], dim=-1)
     y, _ = ssd_chunked_ref(dt, A.to(x.dtype), x.reshape(b, l, h, d_head),
                            Bm.reshape(b, l, n_groups, d_state), Cm.reshape(b, l, n_groups, d_state),
                            D.to(x.dtype) if D is not None else None, chunk=chunk)
-    return rmsnorm_gated_ref(y.reshape(b, l, d_inner), z, norm_w, n_groups, eps)
+    return handover(rmsnorm_gated_ref(handover(y).reshape(b, l, d_inner), z, norm_w, n_groups, eps))

@@ -461,7 +461,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
     M2_REQUIRE(p->ngroups * w.nslices <= 65535, M2_ERR_SHAPE, "ssd_bwd: too many group slices");
     int rc;
     // recompute G (+ operand tiles), S_prev, final state
-    if ((rc = ssd_launch_states<T, P, N>(p, w, w.sfinal, st))) return rc;
+    if ((rc = ssd_launch_states<T, P, N>(p, w, nullptr, st))) return rc;
     // local dS contributions (reuses the `local` region) and the reverse recurrence
     {
         auto k = chunk_state_kernel<T, P, N, true>;
@@ -475,7 +475,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         if ((rc = check_launch("ssd chunk_state_kernel<dstate>"))) return rc;
         state_scan_kernel<T, P * N, true><<<dim3((unsigned)p->nheads, (unsigned)p->batch, kScanSplit), 256, 0, st>>>(
             w.local, w.lam, p->d_final_state, static_cast<T*>(w.dprev), p->d_initial_state,
-            static_cast<const T*>(w.prev), w.sfinal, w.dlam, p->nheads, nc);
+            static_cast<const T*>(w.prev), w.dlam, p->nheads, nc);
         if ((rc = check_launch("ssd state_scan_kernel<reverse>"))) return rc;
     }
     {

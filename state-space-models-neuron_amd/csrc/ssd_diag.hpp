@@ -294,17 +294,25 @@ diag_off_kernel(const DiagArgs a) {
             if (lane == 0) s_red[wave] = dD_loc;
             __syncthreads();      // s_dir, s_rb, s_red complete; also the "tiles are free" barrier for the next head
             if (wave == 0) {
-                // da_j = sum_{i>=j} dl_i + <dS, S_new>;  lanes scan the tokens in reverse order (127-lane, 63-lane)
+                // da_t = sum_{i>=t} (dl_diag_i + dl_c_i) + sum_{j<t} rb_j + dlam;  lanes hold the tokens in reverse
+                // order (127-lane, 63-lane), so the suffix over tokens is an inclusive prefix over lanes and the
+                // exclusive prefix over tokens an exclusive suffix over lanes.
                 const int64_t bhc = (b * a.nheads + h) * a.nchunks + c;
                 const int ta = kQ - 1 - lane, tb = 63 - lane;
-                float xa = a.dl_diag[bhc * kQ + ta] + a.dl_c[bhc * kQ + ta] - s_rb[ta];
-                float xb = a.dl_diag[bhc * kQ + tb] + a.dl_c[bhc * kQ + tb] - s_rb[tb];
+                float xa = a.dl_diag[bhc * kQ + ta] + a.dl_c[bhc * kQ + ta];
+                float xb = a.dl_diag[bhc * kQ + tb] + a.dl_c[bhc * kQ + tb];
+                const float ra = s_rb[ta], rbv = s_rb[tb];
+                float ya = ra, yb = rbv;
 #pragma unroll
                 for (int o = 1; o < 64; o <<= 1) {
                     const float na = __shfl_up(xa, o, 64), nb = __shfl_up(xb, o, 64);
+                    const float ma = __shfl_down(ya, o, 64), mb = __shfl_down(yb, o, 64);
                     if (lane >= o) { xa += na; xb += nb; }
+                    if (lane + o < 64) { ya += ma; yb += mb; }
                 }
                 xb += __shfl(xa, 63, 64);
+                xa += (ya - ra) + __shfl(yb, 0, 64);
+                xb += yb - rbv;
                 float dlm = 0.f;
 #pragma unroll
                 for (int sp = 0; sp < kScanSplit; ++sp) dlm += a.dlam[bhc * kScanSplit + sp];

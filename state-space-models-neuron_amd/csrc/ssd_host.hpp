@@ -6,14 +6,13 @@
 namespace m2 {
 
 // Workspace regions.  Forward uses G, local, prev, lam.  Backward additionally uses
-// sfinal (fp32 final state of the recomputed forward), dprev (gradient w.r.t. the state
-// leaving each chunk, operand type), dlam, dl (per-token gradient of the in-chunk cumulative
+// dprev (gradient w.r.t. the state leaving each chunk, operand type), dlam, dl (per-token gradient of the in-chunk cumulative
 // sum, per head), per-(b,h,chunk) partials of dA and dD, and
 // per-(b,chunk,group,head-slice) fp32 partials of dB and dC.
 struct SsdWorkspace {
     float* G = nullptr; float* local = nullptr; void* prev = nullptr; float* lam = nullptr;
     void* Gm = nullptr; void* Gmt = nullptr; void* Bt = nullptr; void* Ct = nullptr;
-    float* sfinal = nullptr; void* dprev = nullptr; float* dlam = nullptr;
+    void* dprev = nullptr; float* dlam = nullptr;
     float* dAp = nullptr; float* dDp = nullptr; float* dBp = nullptr; float* dCp = nullptr; float* dl = nullptr; float* dlc = nullptr; float* dGp = nullptr;
     float* dGs = nullptr; float* dBs = nullptr; float* dCs = nullptr;   // partials summed over the head slices
     int64_t nslices = 1, heads_per_slice = 1;
@@ -73,7 +72,6 @@ inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd) {
     w.Ct = take(grp * p->dstate * kQ * esz);
     if (bwd) {
         ssd_bwd_slicing(p, &w.nslices, &w.heads_per_slice);
-        w.sfinal = reinterpret_cast<float*>(take((size_t)p->batch * p->nheads * p->headdim * p->dstate * 4));
         w.dprev = take(tiles * esz);
         w.dlam = reinterpret_cast<float*>(take(bhc * 4 * kScanSplit));
         w.dAp = reinterpret_cast<float*>(take(bhc * 4));
@@ -159,7 +157,7 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
     }
     {
         state_scan_kernel<T, P * N, false><<<dim3((unsigned)p->nheads, (unsigned)p->batch, kScanSplit), 256, 0, st>>>(
-            w.local, w.lam, p->initial_state, static_cast<T*>(w.prev), final_out, nullptr, nullptr, nullptr, p->nheads, nc);
+            w.local, w.lam, p->initial_state, static_cast<T*>(w.prev), final_out, nullptr, nullptr, p->nheads, nc);
         if ((rc = check_launch("ssd state_scan_kernel"))) return rc;
     }
     return M2_OK;

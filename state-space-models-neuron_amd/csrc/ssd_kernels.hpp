@@ -189,16 +189,21 @@ chunk_state_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_
 //     run = init;  for c = 0..nc-1:  prev[c] = T(run);  run = e^{lam_c} run + local[c];  final = run
 // reverse (REVERSE == true), the gradient recurrence:
 //     run = dfinal;  for c = nc-1..0:  prev[c] = T(run)   (= dL/dS_new(c));
-//                                      dlam[c][split] = <run, S_new(c)> over this workgroup's part;
+//                                      dlam[c][split] = e^{lam_c} <run, sprev[c]> over this workgroup's part
+//                                      (sprev[c] = the forward state entering chunk c);
 //                                      run = e^{lam_c} run + local[c]
-//     dinit = run.     S_new(c) = sprev[c+1] for c < nc-1, the fp32 final state for c = nc-1.
+//     dinit = run.
+// dlam is the part of dL/dLam_c that flows through the carried state only.  The part through the chunk's own
+// tokens is added by the consumer as a PREFIX sum of per-token terms; forming it here as <run, S_new(c)> and
+// subtracting a suffix sum there would cancel two large numbers rounded differently (operand-type copies of
+// the states), leaving an error that is constant over the chunk and accumulates in dA.
 constexpr int kScanSplit = 4;
 
 template <typename T, int PN, bool REVERSE>
 __global__ void __launch_bounds__(256)
 state_scan_kernel(const float* __restrict__ local, const float* __restrict__ lam, const float* __restrict__ init,
                   T* __restrict__ prev, float* __restrict__ final_out,
-                  const T* __restrict__ sprev, const float* __restrict__ sfinal, float* __restrict__ dlam,
+                  const T* __restrict__ sprev, float* __restrict__ dlam,
                   int64_t nheads, int64_t nchunks) {
     constexpr int EPT = PN / 4 / 256 / kScanSplit;
     static_assert(PN % (1024 * kScanSplit) == 0, "state size must be a multiple of 4096 elements");
@@ -231,29 +236,20 @@ state_scan_kernel(const float* __restrict__ local, const float* __restrict__ lam
             if (sizeof(T) == 2) *reinterpret_cast<uint2*>(prev + tile + off) = *reinterpret_cast<const uint2*>(o);
             else *reinterpret_cast<uint4*>(prev + tile + off) = *reinterpret_cast<const uint4*>(o);
             if (REVERSE) {
-                float sn[4];
-                if (c == nchunks - 1) {
-                    const floatx4 f = *reinterpret_cast<const floatx4*>(sfinal + bh * PN + off);
+                // state that ENTERED this chunk in the forward pass (operand type, as the other kernels consume it)
+                T tv[4];
+                if (sizeof(T) == 2) *reinterpret_cast<uint2*>(tv) = *reinterpret_cast<const uint2*>(sprev + tile + off);
+                else *reinterpret_cast<uint4*>(tv) = *reinterpret_cast<const uint4*>(sprev + tile + off);
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) sn[q] = f[q];
-                } else {
-                    const int64_t nxt = ((b * nchunks + c + 1) * nheads + h) * (int64_t)PN;
-                    T tv[4];
-                    if (sizeof(T) == 2) *reinterpret_cast<uint2*>(tv) = *reinterpret_cast<const uint2*>(sprev + nxt + off);
-                    else *reinterpret_cast<uint4*>(tv) = *reinterpret_cast<const uint4*>(sprev + nxt + off);
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) sn[q] = to_f32(tv[q]);
-                }
-#pragma unroll
-                for (int q = 0; q < 4; ++q) dot += run[e][q] * sn[q];
+                for (int q = 0; q < 4; ++q) dot += run[e][q] * to_f32(tv[q]);
             }
 #pragma unroll
             for (int q = 0; q < 4; ++q) run[e][q] = dec * run[e][q] + loc[q];
         }
         if (REVERSE) {
-            // per-wave partial of <dS, S_new>; the four partials are combined once per kRedBatch chunks so the
-            // streaming loop has no barrier
-            dot = warp_sum(dot);
+            // per-wave partial of e^{Lam} <dS, S_prev>; the four partials are combined once per kRedBatch chunks so
+            // the streaming loop has no barrier
+            dot = warp_sum(dot) * dec;
             if (lane == 0) red[(cc % kRedBatch) * 4 + wave] = dot;
             if ((cc % kRedBatch) == kRedBatch - 1 || cc == nchunks - 1) {
                 __syncthreads();
