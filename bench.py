@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X Mamba-2 mixer hot path.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|ssd|conv|decode] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|ssd|conv|decode|copy] [--no-cpu]
 
 One "step" is one pass of the hot path over one batch of synthetic input, inputs resident in HBM:
   ssd    : SSD chunked scan fwd+bwd, bf16, 2.7B shape (b4, l2048, h80, p64, n128, g1, chunk 128)   <- headline
@@ -132,6 +132,33 @@ def bench_decode(steps, warmup):
                           "algorithmic_bytes_per_step": bytes_, "kernels": "decode_conv_kernel + decode_ssm_kernel, 64 launches each"})
 
 
+def bench_copy(steps, warmup):
+    """Plain 16-byte-per-lane copy kernel over 1 GiB (read 1 GiB + write 1 GiB per launch): the HBM rate a trivial
+    streaming kernel reaches on this box, and the dispatch of known size the HBM-traffic counters are scaled by."""
+    import torch
+    from mamba2 import _lib
+    lib = _lib.load()
+    nbytes = 1 << 30
+    bufs = [(torch.empty(nbytes, dtype=torch.uint8, device="cuda:0").fill_(i), torch.empty(nbytes, dtype=torch.uint8, device="cuda:0")) for i in range(2)]
+    state = {"i": 0}
+
+    def step():
+        src, dst = bufs[state["i"] % 2]
+        state["i"] += 1
+        rc = lib.m2_stream_copy(src.data_ptr(), dst.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+        if rc != 0:
+            raise RuntimeError(lib.m2_last_error().decode())
+
+    _, per = event_time_ms(step, steps, warmup)
+    ms = sum(per) / len(per)
+    moved = 2 * nbytes
+    return dict(metric="plain copy kernel HBM rate", value=moved / (ms * 1e-3) / 1e9, unit="GB/s", ms_per_step=ms, dtype="u8",
+                config={"workload": "stream_copy_kernel, 1 GiB read + 1 GiB write per launch"},
+                roofline={"bound": "hbm", "achieved": moved / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_step": moved,
+                          "kernels": "stream_copy_kernel"})
+
+
 def cpu_baseline_ssd():
     """The pure-PyTorch chunked oracle (fp32, autograd) on the host cores: the full headline configuration."""
     import torch
@@ -156,7 +183,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", choices=["all", "ssd", "conv", "decode"])
+    ap.add_argument("--workload", default="all", choices=["all", "ssd", "conv", "decode", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -189,8 +216,10 @@ def main():
         other["conv1d"] = bench_conv(a.steps, a.warmup)
     if a.workload in ("all", "decode"):
         other["decode"] = bench_decode(max(3, a.steps // 4), max(1, a.warmup // 2))
+    if a.workload in ("all", "copy"):
+        other["stream_copy"] = bench_copy(a.steps, a.warmup)
     if a.workload not in ("all", "ssd"):
-        key = "conv1d" if a.workload == "conv" else "decode"
+        key = {"conv": "conv1d", "decode": "decode", "copy": "stream_copy"}[a.workload]
         out.update(other.pop(key))
         out.update({"n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "scaling": "weak", "vs_baseline": None, "data": "synthetic"})
         out.setdefault("higher_is_better", True)
