@@ -57,14 +57,16 @@ def event_time_ms(fn, steps, warmup):
 
 def bench_ssd(steps, warmup):
     import torch
-    from mamba2.mamba2_kernel import ssd_backward, ssd_forward
+    from mamba2.mamba2_kernel import SAVE_CHUNK_STATES, alloc_chunk_states, ssd_backward, ssd_forward
     from oracle.ssd import make_ssd_inputs
     cfg = SSD_CFG
     d = make_ssd_inputs(cfg["b"], cfg["l"], cfg["h"], cfg["p"], cfg["n"], cfg["g"], seed=0, dtype=torch.bfloat16, device="cuda:0")
+    # what Mamba2Kernel.forward/backward do: the forward keeps the chunk states for the backward (84 MB here)
+    states = alloc_chunk_states(d["X"], d["B"]) if SAVE_CHUNK_STATES else None
 
     def step():
-        y, _ = ssd_forward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"])
-        ssd_backward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], d["dy"])
+        y, _ = ssd_forward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], chunk_states=states)
+        ssd_backward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], d["dy"], chunk_states=states)
 
     wall_ms, per = event_time_ms(step, steps, warmup)
     per.sort()

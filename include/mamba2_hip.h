@@ -87,14 +87,21 @@ int m2_conv1d_bwd(const m2_conv1d_params* p, void* stream);
  * dt (b,l,h), A (h) fp32, x (b,l,h,p), B,C (b,l,g,n), D (h) fp32 or NULL,
  * initial_state / final_state (b,h,p,n) fp32 contiguous or NULL, y (b,l,h,p).
  * Supported: p in {64,128}, n in {64,128}, h % g == 0, any l >= 0, any b >= 0.
- * Backward takes the same inputs plus dy (it recomputes per chunk; y is unused) and writes
+ * Backward takes the same inputs plus dy (y is unused) and writes
  * dx, ddt, dB, dC in the dtype of the matching input and dA (h), dD (h) in fp32,
  * already summed over the batch (the reference sums them in its wrapper,
  * mamba2_kernel.py:514).
+ * chunk_states (optional): (b, ceil(l/128), h, p, n) elements of `dtype`,
+ * m2_ssd_chunk_states_bytes() bytes, 16-byte aligned -- the SSM state entering each chunk.
+ * Forward: if non-NULL it is written there (otherwise into the workspace).  Backward: if
+ * non-NULL it must hold what the forward wrote for the same inputs and is read instead of
+ * being recomputed; with NULL the backward recomputes it from the inputs, as the reference
+ * does (mamba2_kernel.py:363-367).
  */
 typedef struct m2_ssd_params {
     const void* x; const void* dt; const float* A; const void* B; const void* C; const float* D;
     const float* initial_state; float* final_state;
+    void* chunk_states;                                 /* optional, see above          */
     void* y;                                            /* fwd: out; unused by bwd      */
     /* backward only */
     const void* dy; const float* d_final_state;
@@ -115,6 +122,7 @@ typedef struct m2_ssd_params {
     int32_t dt_dtype;                                   /* dt, ddt                      */
 } m2_ssd_params;
 
+size_t m2_ssd_chunk_states_bytes(const m2_ssd_params* p);
 size_t m2_ssd_fwd_workspace_bytes(const m2_ssd_params* p);
 int m2_ssd_fwd(const m2_ssd_params* p, void* stream);
 size_t m2_ssd_bwd_workspace_bytes(const m2_ssd_params* p);

@@ -460,8 +460,8 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
     const dim3 grid_s((unsigned)nc, (unsigned)(p->ngroups * w.nslices), (unsigned)p->batch);
     M2_REQUIRE(p->ngroups * w.nslices <= 65535, M2_ERR_SHAPE, "ssd_bwd: too many group slices");
     int rc;
-    // recompute G (+ operand tiles), S_prev, final state
-    if ((rc = ssd_launch_states<T, P, N>(p, w, nullptr, st))) return rc;
+    // G (+ operand tiles); the state entering each chunk, unless the caller kept the forward's
+    if ((rc = ssd_launch_states<T, P, N>(p, w, nullptr, st, p->chunk_states != nullptr))) return rc;
     // local dS contributions (reuses the `local` region) and the reverse recurrence
     {
         auto k = chunk_state_kernel<T, P, N, true>;
@@ -470,7 +470,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         int64_t ns, hps;
         ssd_head_slicing(p, 1024, &ns, &hps);
         k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * ns), (unsigned)p->batch), 256, sm, st>>>(
-            dy, p->dt, dt_f32, p->A, static_cast<const T*>(w.Ct), w.local, nullptr, p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
+            dy, p->dt, dt_f32, p->A, static_cast<const T*>(w.Ct), w.local, w.lam, p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
             p->dy_stride_b, p->dy_stride_l, p->dy_stride_h, p->dt_stride_b, p->dt_stride_l);
         if ((rc = check_launch("ssd chunk_state_kernel<dstate>"))) return rc;
         state_scan_kernel<T, P * N, true><<<dim3((unsigned)p->nheads, (unsigned)p->batch, kScanSplit), 256, 0, st>>>(

@@ -63,7 +63,8 @@ inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd) {
     auto take = [&](size_t n) { unsigned char* r = b8 ? b8 + off : nullptr; off += align_up(n, 256); return r; };
     w.G = reinterpret_cast<float*>(take((size_t)p->batch * nc * p->ngroups * kQ * kQ * 4));
     w.local = reinterpret_cast<float*>(take(tiles * 4));
-    w.prev = take(tiles * esz);
+    if (p->chunk_states) w.prev = p->chunk_states;      // caller keeps the chunk states (forward -> backward)
+    else w.prev = take(tiles * esz);
     w.lam = reinterpret_cast<float*>(take(bhc * 4));
     const size_t grp = (size_t)p->batch * nc * p->ngroups;
     w.Gm = take(grp * kQ * kQ * esz);
@@ -107,6 +108,7 @@ inline int ssd_check(const m2_ssd_params* p, const char* who) {
                p->C_stride_b % V == 0 && p->C_stride_l % V == 0 && p->C_stride_g % V == 0,
                M2_ERR_ALIGN, "%s: x/B/C strides must be multiples of %d elements (16 bytes)", who, V);
     M2_REQUIRE(aligned16(p->x) && aligned16(p->B) && aligned16(p->C), M2_ERR_ALIGN, "%s: x/B/C must be 16-byte aligned", who);
+    M2_REQUIRE(aligned16(p->chunk_states), M2_ERR_ALIGN, "%s: chunk_states must be 16-byte aligned", who);
     return M2_OK;
 }
 
@@ -125,9 +127,10 @@ inline size_t state_smem() { return (size_t)(P + N) * lds_ld<T>(kQ) * sizeof(T);
 template <typename T>
 inline size_t cb_smem() { return (size_t)2 * kQ * lds_ld<T>(64) * sizeof(T); }
 
-// G = C B^T, local chunk states, forward state scan.  Used by the forward and (recompute) by the backward.
+// G = C B^T, local chunk states, forward state scan.  Used by the forward and (recompute) by the backward;
+// `cb_only` stops after the first (the backward was handed the chunk states).
 template <typename T, int P, int N>
-inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, float* final_out, hipStream_t st) {
+inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, float* final_out, hipStream_t st, bool cb_only = false) {
     const int64_t nc = ceil_div(p->seqlen, (int64_t)kQ);
     const T* x = static_cast<const T*>(p->x);
     const T* Bm = static_cast<const T*>(p->B);
@@ -143,6 +146,7 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
             p->C_stride_b, p->C_stride_l, p->C_stride_g);
         if ((rc = check_launch("ssd cb_kernel"))) return rc;
     }
+    if (cb_only) return M2_OK;
     {
         auto k = chunk_state_kernel<T, P, N, false>;
         const size_t sm = state_smem<T, P, N>();

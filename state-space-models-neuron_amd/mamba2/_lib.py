@@ -31,7 +31,7 @@ class Conv1dParams(C.Structure):
 
 class SsdParams(C.Structure):
     _fields_ = [("x", _vp), ("dt", _vp), ("A", _vp), ("B", _vp), ("C", _vp), ("D", _vp),
-                ("initial_state", _vp), ("final_state", _vp), ("y", _vp),
+                ("initial_state", _vp), ("final_state", _vp), ("chunk_states", _vp), ("y", _vp),
                 ("dy", _vp), ("d_final_state", _vp),
                 ("dx", _vp), ("ddt", _vp), ("dA", _vp), ("dB", _vp), ("dC", _vp), ("dD", _vp), ("d_initial_state", _vp),
                 ("workspace", _vp), ("workspace_bytes", _sz),
@@ -66,6 +66,7 @@ SYMBOLS = {
     "m2_conv1d_fwd": (C.c_int, [C.POINTER(Conv1dParams), _vp]),
     "m2_conv1d_bwd_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
     "m2_conv1d_bwd": (C.c_int, [C.POINTER(Conv1dParams), _vp]),
+    "m2_ssd_chunk_states_bytes": (_sz, [C.POINTER(SsdParams)]),
     "m2_ssd_fwd_workspace_bytes": (_sz, [C.POINTER(SsdParams)]),
     "m2_ssd_fwd": (C.c_int, [C.POINTER(SsdParams), _vp]),
     "m2_ssd_bwd_workspace_bytes": (_sz, [C.POINTER(SsdParams)]),

@@ -17,7 +17,7 @@ import torch
 
 from . import glue
 from .conv1d_grouped import conv1d_backward, conv1d_forward
-from .mamba2_kernel import ssd_backward, ssd_forward
+from .mamba2_kernel import alloc_chunk_states, ssd_backward, ssd_forward
 
 NORM_EPS = 1e-5     # fixed in the reference's fused kernel (fused_kernel.py:254)
 
@@ -43,20 +43,22 @@ def _xbc_views(conv_out, n_groups, d_state, d_inner, d_head):
     return x, Bm, Cm
 
 
-def _forward_parts(zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, n_groups, d_state, d_inner, d_head):
+def _forward_parts(zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, n_groups, d_state, d_inner, d_head, keep_states=False):
     z, xBC, dt, h, d_conv = _views(zxBCdt, n_groups, d_state, d_inner, d_head)
     b, l, _ = zxBCdt.shape
     conv_out = torch.empty((b, l, d_conv), dtype=zxBCdt.dtype, device=zxBCdt.device)
     conv1d_forward(xBC, conv_w, conv_b, "silu", channels_last=True, out=conv_out)
     dt_sp = glue.softplus_bias(dt, dt_bias)
     x, Bm, Cm = _xbc_views(conv_out, n_groups, d_state, d_inner, d_head)
-    y, _ = ssd_forward(dt_sp, logA, x, Bm, Cm, D)
+    # the scan's chunk states are kept for the backward when one follows directly (no second recompute there)
+    states = alloc_chunk_states(x, Bm) if (keep_states and x.numel() > 0) else None
+    y, _ = ssd_forward(dt_sp, logA, x, Bm, Cm, D, chunk_states=states)
     scan_out = y.view(b, l, d_inner)
     norm_out = glue.rmsnorm_gated(scan_out, z, norm_w, n_groups, NORM_EPS, out_dtype=zxBCdt.dtype)
-    return norm_out, conv_out, dt_sp, scan_out
+    return norm_out, conv_out, dt_sp, scan_out, states
 
 
-def _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out,
+def _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out, states,
                     n_groups, d_state, d_inner, d_head):
     z, xBC, dt, h, d_conv = _views(zxBCdt, n_groups, d_state, d_inner, d_head)
     b, l, width = zxBCdt.shape
@@ -71,7 +73,7 @@ def _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, 
     d_conv_out = torch.empty_like(conv_out)
     dx_v, dB_v, dC_v = _xbc_views(d_conv_out, n_groups, d_state, d_inner, d_head)
     d_dt_sp, d_logA, _, _, _, d_D, _ = ssd_backward(dt_sp, logA, x, Bm, Cm, D, d_scan_out.view(b, l, h, d_head),
-                                                     out_dX=dx_v, out_dB=dB_v, out_dC=dC_v)
+                                                     out_dX=dx_v, out_dB=dB_v, out_dC=dC_v, chunk_states=states)
     # softplus backward (into the dt columns) and conv backward (into the xBC columns)
     d_dt_bias = glue.softplus_bias_bwd(dt, dt_bias, d_dt_sp, out_d_in=ddt_view)
     _, d_conv_w, d_conv_b = conv1d_backward(xBC, conv_w, conv_b, d_conv_out, "silu", channels_last=True, out_dx=dxBC_view)
@@ -93,8 +95,10 @@ class Mamba2FusedKernel(torch.autograd.Function):
     def backward(ctx, d_output):
         zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w = ctx.saved_tensors
         # recompute conv, softplus and scan (only the inputs were saved)
-        _, conv_out, dt_sp, scan_out = _forward_parts(zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, *ctx.dims)
-        grads = _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out, *ctx.dims)
+        _, conv_out, dt_sp, scan_out, states = _forward_parts(zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, *ctx.dims,
+                                                              keep_states=True)
+        grads = _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out, states,
+                                *ctx.dims)
         return (*grads, None, None, None, None)
 
 
@@ -102,16 +106,19 @@ class Mamba2FusedKernelWithCaching(torch.autograd.Function):
     @staticmethod
     def forward(ctx, zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias,
                 norm_weight, n_groups, ssm_state_size, intermediate_size, head_dim):
-        norm_out, conv_out, dt_sp, scan_out = _forward_parts(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias, norm_weight,
-                                                             n_groups, ssm_state_size, intermediate_size, head_dim)
+        norm_out, conv_out, dt_sp, scan_out, states = _forward_parts(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias,
+                                                                     norm_weight, n_groups, ssm_state_size, intermediate_size,
+                                                                     head_dim, keep_states=True)
         ctx.dims = (n_groups, ssm_state_size, intermediate_size, head_dim)
+        ctx.chunk_states = states
         ctx.save_for_backward(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias, norm_weight, conv_out, dt_sp, scan_out)
         return norm_out
 
     @staticmethod
     def backward(ctx, d_output):
         zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out = ctx.saved_tensors
-        grads = _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out, *ctx.dims)
+        grads = _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out,
+                                ctx.chunk_states, *ctx.dims)
         return (*grads, None, None, None, None)
 
 

@@ -7,6 +7,8 @@ Extensions (keyword-only, default off): ``initial_state`` (b,h,p,n) fp32 and
 ``return_final_state`` -> (Y, S[b,h,p,n] fp32).  X, B, C may be strided views into a packed
 [x | B | C] buffer as long as their innermost dimension is contiguous.
 """
+import os
+
 import torch
 
 from . import _lib
@@ -58,7 +60,14 @@ def _validate(dt, A, X, B, C, D, initial_state):
     _lib.require_gpu(dt, A, X, B, C, D, initial_state)
 
 
-def ssd_forward(dt, A, X, B, C, D=None, initial_state=None, want_final_state=False):
+def alloc_chunk_states(X, B):
+    """Buffer for the SSM state entering each 128-token chunk, (b, ceil(l/128), h, p, n) in X's dtype:
+    filled by ``ssd_forward(..., chunk_states=buf)`` and consumed by ``ssd_backward(..., chunk_states=buf)``."""
+    b, l, h, hd = X.shape
+    return torch.empty((b, -(-l // 128), h, hd, B.shape[3]), dtype=X.dtype, device=X.device)
+
+
+def ssd_forward(dt, A, X, B, C, D=None, initial_state=None, want_final_state=False, chunk_states=None):
     """Raw forward through the C ABI.  Returns (Y, final_state or None)."""
     _validate(dt, A, X, B, C, D, initial_state)
     lib = _lib.load()
@@ -72,6 +81,7 @@ def ssd_forward(dt, A, X, B, C, D=None, initial_state=None, want_final_state=Fal
     p = SsdParams()
     _fill_common(p, dt, A32, X, B, C, D32)
     p.initial_state, p.final_state, p.y = ptr(S0), ptr(S), ptr(Y)
+    p.chunk_states = _chunk_states_ptr(lib, p, chunk_states)
     p.y_stride_b, p.y_stride_l, p.y_stride_h = _strides3(Y)
     nbytes = lib.m2_ssd_fwd_workspace_bytes(p)
     ws = _lib.Workspace.get(nbytes, X.device)
@@ -81,12 +91,22 @@ def ssd_forward(dt, A, X, B, C, D=None, initial_state=None, want_final_state=Fal
     return Y, S
 
 
+def _chunk_states_ptr(lib, p, chunk_states):
+    if chunk_states is None:
+        return None
+    need = lib.m2_ssd_chunk_states_bytes(p)
+    if not chunk_states.is_contiguous() or chunk_states.numel() * chunk_states.element_size() != need or \
+            _lib.dtype_code(chunk_states.dtype) != p.dtype:
+        raise ValueError(f"chunk_states must be a contiguous buffer of {need} bytes in the dtype of X (see alloc_chunk_states)")
+    return ptr(chunk_states)
+
+
 def ssd_backward(dt, A, X, B, C, D, dY, initial_state=None, d_final_state=None, want_dinitial=False,
-                 out_dX=None, out_dB=None, out_dC=None):
+                 out_dX=None, out_dB=None, out_dC=None, chunk_states=None):
     """Raw backward through the C ABI.
     Returns (ddt, dA fp32 (h), dX, dB, dC, dD fp32 (h) or None, d_initial_state or None).
     ``out_dX/out_dB/out_dC`` let the caller provide (strided) destinations, e.g. views of a packed
-    [dx | dB | dC] buffer."""
+    [dx | dB | dC] buffer.  ``chunk_states``: what the forward wrote for the same inputs (skips the recompute)."""
     lib = _lib.load()
     b, l, h, hd = X.shape
     g, n = B.shape[2], B.shape[3]
@@ -110,6 +130,7 @@ def ssd_backward(dt, A, X, B, C, D, dY, initial_state=None, d_final_state=None, 
     p = SsdParams()
     _fill_common(p, dt, A32, X, B, C, D32)
     p.initial_state, p.dy, p.d_final_state = ptr(S0), ptr(dY), ptr(dSf)
+    p.chunk_states = _chunk_states_ptr(lib, p, chunk_states)
     p.dx, p.ddt, p.dA, p.dB, p.dC, p.dD, p.d_initial_state = ptr(dX), ptr(ddt), ptr(dA), ptr(dB), ptr(dC), ptr(dD), ptr(dS0)
     p.dy_stride_b, p.dy_stride_l, p.dy_stride_h = _strides3(dY)
     p.dx_stride_b, p.dx_stride_l, p.dx_stride_h = _strides3(dX)
@@ -124,6 +145,13 @@ def ssd_backward(dt, A, X, B, C, D, dY, initial_state=None, d_final_state=None, 
     return ddt, dA, dX, dB, dC, dD, dS0
 
 
+# The reference saves only the inputs and recomputes the chunk states in the backward
+# (``mamba2/mamba2_kernel.py:492,363-367``) because its device memory is scarce.  With 288 GB of HBM the
+# states entering each chunk (as many bytes as X) are kept instead, which removes two kernels and
+# ~0.5 GB of traffic from the backward at the 2.7B shape.  M2_SSD_SAVE_STATES=0 restores recompute.
+SAVE_CHUNK_STATES = os.environ.get("M2_SSD_SAVE_STATES", "1") != "0"
+
+
 class Mamba2Kernel(torch.autograd.Function):
     """forward(ctx, dt, A, X, B, C, D) -> Y; backward -> (ddt, dA, dX, dB, dC, dD)
     (``mamba2/mamba2_kernel.py:490,498,515``).  Two optional trailing arguments carry the
@@ -131,8 +159,10 @@ class Mamba2Kernel(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, dt, A, X, B, C, D, initial_state=None, return_final_state=False):
-        Y, S = ssd_forward(dt, A, X, B, C, D, initial_state, return_final_state)
-        # only the inputs are saved, as in the reference (:492); the backward recomputes per chunk
+        needs_grad = any(ctx.needs_input_grad[:7])
+        states = alloc_chunk_states(X, B) if (SAVE_CHUNK_STATES and needs_grad and X.numel() > 0) else None
+        Y, S = ssd_forward(dt, A, X, B, C, D, initial_state, return_final_state, chunk_states=states)
+        ctx.chunk_states = states
         ctx.save_for_backward(dt, A, X, B, C, D, initial_state)
         ctx.return_final_state = return_final_state
         if return_final_state:
@@ -144,7 +174,9 @@ class Mamba2Kernel(torch.autograd.Function):
         dt, A, X, B, C, D, initial_state = ctx.saved_tensors
         dS = rest[0] if (ctx.return_final_state and rest and rest[0] is not None) else None
         want_dinit = initial_state is not None and ctx.needs_input_grad[6]
-        ddt, dA, dX, dB, dC, dD, dS0 = ssd_backward(dt, A, X, B, C, D, d_output, initial_state, dS, want_dinit)
+        ddt, dA, dX, dB, dC, dD, dS0 = ssd_backward(dt, A, X, B, C, D, d_output, initial_state, dS, want_dinit,
+                                                     chunk_states=ctx.chunk_states)
+        ctx.chunk_states = None
         dA = dA.to(A.dtype)
         dD = dD.to(D.dtype) if D is not None else None
         return ddt, dA, dX, dB, dC, dD, dS0, None

@@ -155,3 +155,24 @@ def test_ssd_backward_states(dtype):
         e = metric(leaves[key].grad, ref[name])
         assert e < tol, f"{name}: {e}"
     assert metric(S0d.grad, ref["dinitial_state"]) < tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ssd_backward_kept_chunk_states_equal_recompute(dtype):
+    # the backward handed the forward's chunk states must give exactly what the recomputing backward gives
+    from mamba2.mamba2_kernel import alloc_chunk_states, ssd_backward, ssd_forward
+    b, l, h, p, n, g = 2, 300, 4, 64, 128, 2
+    d = _dev(make_ssd_inputs(b, l, h, p, n, g, seed=21, dtype=dtype))
+    S0 = 0.1 * torch.randn(b, h, p, n, generator=torch.Generator().manual_seed(5)).to(DEV)
+    states = alloc_chunk_states(d["X"], d["B"])
+    assert states.shape == (b, 3, h, p, n) and states.dtype == dtype
+    y1, _ = ssd_forward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], S0, chunk_states=states)
+    y0, _ = ssd_forward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], S0)
+    assert torch.equal(y0, y1)
+    assert torch.equal(states[:, 0].float(), S0.to(dtype).float())      # the state entering chunk 0 is the initial state
+    g0 = ssd_backward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], d["dy"], S0, want_dinitial=True)
+    g1 = ssd_backward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], d["dy"], S0, want_dinitial=True, chunk_states=states)
+    for a_, b_ in zip(g0, g1):
+        assert torch.equal(a_, b_)
+    with pytest.raises(ValueError, match="chunk_states"):
+        ssd_backward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], d["dy"], chunk_states=states[:, :2].contiguous())
