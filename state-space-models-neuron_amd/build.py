@@ -17,7 +17,7 @@ OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "mamba2", "libmamba2_hip.so")
 SOURCES = ["api.hip", "conv1d.hip", "decode.hip", "glue.hip", "ssd_fwd.hip", "ssd_bwd.hip"]
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
-         "-Wno-unused-command-line-argument",
+         "-Wno-unused-command-line-argument", "-Wno-inline-asm",
          # packed-FP32 VALU forms are kept out of the generated code
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 

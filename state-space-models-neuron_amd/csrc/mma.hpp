@@ -212,9 +212,10 @@ __device__ __forceinline__ float half_wave_reduce16(float (&v)[16], int* reg_ind
 
 // Wave-private chunk cumulative sum: every wave computes l for all 128 tokens by itself (lane holds tokens
 // `lane` and `lane + 64`), so no block barrier is needed.  Tokens >= valid behave as dt = 0.
+// Split in two so that the loads of the next head's dt can be issued long before they are needed.
 template <typename T>
-__device__ __forceinline__ void wave_chunk_cumsum(const void* __restrict__ dt, int dt_f32, int64_t off, int64_t stride_l,
-                                                  int valid, float A, float& l0, float& l1, float& d0, float& d1) {
+__device__ __forceinline__ void wave_dt_load(const void* __restrict__ dt, int dt_f32, int64_t off, int64_t stride_l,
+                                             int valid, float& d0, float& d1) {
     const int lane = threadIdx.x & 63;
     d0 = 0.f; d1 = 0.f;
     if (dt_f32) {
@@ -226,6 +227,38 @@ __device__ __forceinline__ void wave_chunk_cumsum(const void* __restrict__ dt, i
         if (lane < valid) d0 = to_f32(p[(int64_t)lane * stride_l]);
         if (lane + 64 < valid) d1 = to_f32(p[(int64_t)(lane + 64) * stride_l]);
     }
+}
+// The same loads without conversion or divergent branches (addresses of tokens >= valid are clamped), so that
+// nothing forces a wait for them where they are issued; wave_dt_cvt turns them into dt values where they are used.
+template <typename T>
+__device__ __forceinline__ void wave_dt_load_raw(const void* __restrict__ dt, int dt_f32, int64_t off, int64_t stride_l,
+                                                 int valid, uint32_t& r0, uint32_t& r1) {
+    const int lane = threadIdx.x & 63;
+    const int t0 = lane < valid ? lane : valid - 1, t1 = lane + 64 < valid ? lane + 64 : valid - 1;
+    if (dt_f32) {
+        const uint32_t* p = static_cast<const uint32_t*>(dt) + off;
+        r0 = p[(int64_t)t0 * stride_l]; r1 = p[(int64_t)t1 * stride_l];
+    } else {
+        static_assert(sizeof(T) == 2 || sizeof(T) == 4, "dt element size");
+        if (sizeof(T) == 2) {
+            const uint16_t* p = static_cast<const uint16_t*>(dt) + off;
+            r0 = p[(int64_t)t0 * stride_l]; r1 = p[(int64_t)t1 * stride_l];
+        } else {
+            const uint32_t* p = static_cast<const uint32_t*>(dt) + off;
+            r0 = p[(int64_t)t0 * stride_l]; r1 = p[(int64_t)t1 * stride_l];
+        }
+    }
+}
+template <typename T>
+__device__ __forceinline__ void wave_dt_cvt(int dt_f32, int valid, uint32_t r0, uint32_t r1, float& d0, float& d1) {
+    const int lane = threadIdx.x & 63;
+    if (dt_f32 || sizeof(T) == 4) { d0 = __uint_as_float(r0); d1 = __uint_as_float(r1); }
+    else { d0 = __uint_as_float(r0 << 16); d1 = __uint_as_float(r1 << 16); }      // bf16 bits -> fp32
+    if (lane >= valid) d0 = 0.f;
+    if (lane + 64 >= valid) d1 = 0.f;
+}
+__device__ __forceinline__ void wave_cumsum_from(float A, float d0, float d1, float& l0, float& l1) {
+    const int lane = threadIdx.x & 63;
     l0 = A * d0; l1 = A * d1;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
@@ -233,6 +266,21 @@ __device__ __forceinline__ void wave_chunk_cumsum(const void* __restrict__ dt, i
         if (lane >= o) { l0 += n0; l1 += n1; }
     }
     l1 += __shfl(l0, 63, 64);
+}
+template <typename T>
+__device__ __forceinline__ void wave_chunk_cumsum(const void* __restrict__ dt, int dt_f32, int64_t off, int64_t stride_l,
+                                                  int valid, float A, float& l0, float& l1, float& d0, float& d1) {
+    wave_dt_load<T>(dt, dt_f32, off, stride_l, valid, d0, d1);
+    wave_cumsum_from(A, d0, d1, l0, l1);
+}
+
+// Orders this wave's LDS writes before its later LDS reads of what OTHER lanes of the same wave wrote
+// (wave-private staging buffers).  The hardware executes one wave's LDS operations in order; the fences
+// keep the compiler from reordering them.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // Inclusive cumulative sum l[t] = sum_{s<=t} A * dt[s] over one chunk (kQ = 128 tokens), in fp32.

@@ -13,6 +13,7 @@
 // Extensions over the reference kernel: optional initial state, final-state output, any batch,
 // ragged sequence length (tokens past the end behave as dt = 0 and are never written).
 #include "ssd_host.hpp"
+#include "ssd_y.hpp"
 
 namespace m2 {
 namespace {
@@ -130,11 +131,19 @@ int ssd_fwd_impl(const m2_ssd_params* p, hipStream_t st) {
     a.seqlen = p->seqlen; a.nheads = p->nheads; a.ngroups = p->ngroups; a.nchunks = nc;
     ssd_head_slicing(p, 1024, &a.nslices, &a.hps);
     a.Y = p->y; a.Y_sb = p->y_stride_b; a.Y_sl = p->y_stride_l; a.Y_sh = p->y_stride_h;
+    M2_REQUIRE(p->ngroups * a.nslices <= 65535, M2_ERR_SHAPE, "ssd_fwd: too many group slices");
+    const dim3 grid((unsigned)nc, (unsigned)(p->ngroups * a.nslices), (unsigned)p->batch);
+    if constexpr (sizeof(T) == 2 && y16_smem<P, N>() <= 160 * 1024) {
+        auto k = ssd_y16_kernel<T, P, N>;
+        const size_t sm = y16_smem<P, N>();
+        if ((rc = allow_smem(k, sm))) return rc;
+        k<<<grid, 256, sm, st>>>(a);
+        return check_launch("ssd_y16_kernel");
+    }
     auto k = diag_off_kernel<T, P, N, false>;
     const size_t sm = diag_smem<T, P, N, false>();
     if ((rc = allow_smem(k, sm))) return rc;
-    M2_REQUIRE(p->ngroups * a.nslices <= 65535, M2_ERR_SHAPE, "ssd_fwd: too many group slices");
-    k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * a.nslices), (unsigned)p->batch), 256, sm, st>>>(a);
+    k<<<grid, 256, sm, st>>>(a);
     return check_launch("ssd diag_off_kernel<fwd>");
 }
 
@@ -167,7 +176,11 @@ extern "C" int m2_ssd_fwd(const m2_ssd_params* p, void* stream) {
         return M2_OK;
     }
     M2_REQUIRE(p->x && p->dt && p->A && p->B && p->C && p->y, M2_ERR_NULL, "ssd_fwd: x, dt, A, B, C, y are required");
-    M2_REQUIRE(p->y_stride_l % 1 == 0, M2_ERR_SHAPE, "ssd_fwd: bad y stride");
+    {
+        const int V = p->dtype == M2_F32 ? 4 : 8;
+        M2_REQUIRE(aligned16(p->y) && p->y_stride_b % V == 0 && p->y_stride_l % V == 0 && p->y_stride_h % V == 0, M2_ERR_ALIGN,
+                   "ssd_fwd: y and its strides must be 16-byte aligned (multiples of %d elements)", V);
+    }
     const size_t need = m2_ssd_fwd_workspace_bytes(p);
     M2_REQUIRE(p->workspace && p->workspace_bytes >= need, M2_ERR_WORKSPACE, "ssd_fwd: workspace %zu bytes < %zu needed",
                p->workspace_bytes, need);

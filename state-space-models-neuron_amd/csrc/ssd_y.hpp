@@ -1,0 +1,260 @@
+// SSD forward output kernel for 16-bit operands, software-pipelined over the heads of a group.
+//
+//     y[i][p] = u_i * ( e^{l_ref} sum_n C[i][n] S_prev[p][n]  +  sum_{j<=i} (G[i][j] v_j) x[j][p] )  +  D x[i][p]
+//
+// (same factorised decay as ssd_diag.hpp: u_i = e^{l_i - l_ref}, v_j = e^{l_ref - l_j} dt_j per 32-token row block,
+// exact per-element fallback when a block's range exceeds kMaxRange).
+//
+// A workgroup (4 waves, wave w owns token rows 32w..32w+31) handles one chunk of one group and loops over `hps`
+// heads.  The two tiles a head needs -- S_prev [P][N] and x [128][P] -- are copied global -> LDS by the
+// asynchronous direct-to-LDS loads of gfx950 (no registers involved) into one of two buffers, ONE HEAD AHEAD:
+// the copy for head k+1 is issued right after the barrier that opens head k and flies while head k's MFMAs and
+// epilogue run.  There is one barrier per head.  Both tiles keep their natural (global) layout in LDS:
+//   * S_prev rows are the MFMA B operand as they are (k = n contiguous);
+//   * x is needed with k = token contiguous; the LDS transpose read (ds_read_b64_tr_b16) delivers exactly that
+//     from the row-major tile, and the epilogue reads the same tile row-wise for the D x term.
+// A direct-to-LDS load writes the 64 lanes' 16-byte pieces to 64 CONSECUTIVE LDS slots, so padding rows is not
+// possible; bank conflicts are avoided by an XOR swizzle of the slot index inside each row instead (each lane
+// simply fetches the global piece that belongs in its slot).
+// The head-independent operands stay in registers for the whole loop: the causal C B^T fragments and the C row
+// fragments.  The epilogue goes through a small wave-private fp32 LDS tile so that y leaves in 16-byte
+// row-contiguous stores, rounded once.
+#pragma once
+#include "ssd_diag.hpp"
+
+namespace m2 {
+
+#define M2_LDS __attribute__((address_space(3)))
+#define M2_GLB __attribute__((address_space(1)))
+
+// wait until this wave's outstanding vector-memory operations (including direct-to-LDS loads) are done;
+// the export and LDS/scalar counters are left alone.  gfx9 encoding: vmcnt = simm16[15:14,3:0], expcnt [6:4],
+// lgkmcnt [11:8].
+__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+// Asynchronous 16-byte-per-lane copy global -> LDS: lane i's 16 bytes land at lds_base + 16 i (lds_base wave-uniform).
+// Written as inline assembly on purpose: for the compiler's own direct-to-LDS builtin the wait-count pass
+// makes every later LDS store (and transpose read) wait for ALL outstanding vector-memory operations, which
+// serialises exactly the copy/compute overlap this is for.  Completion is awaited explicitly (wait_vmem_all) before
+// the barrier that publishes the tile; operations the compiler does not know about can only make its own
+// vmcnt waits more conservative, never too short (vmcnt retires in order).
+__device__ __forceinline__ void async_copy16(const void* gsrc, void* lds_base) {
+    const uint32_t l = __builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(M2_LDS void*)lds_base);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gsrc), "s"(l) : "memory", "m0");
+}
+
+// 16-byte slot s of row `row` lives at slot (s ^ swz) of that row
+template <int SPR> __device__ __forceinline__ int swz_s(int row) { return row & (SPR - 1); }          // S_prev tile
+__device__ __forceinline__ int swz_x(int row) { return ((row >> 1) & 1) << 2; }                      // x tile
+
+template <int P, int N>
+constexpr size_t y16_smem() {
+    return (size_t)2 * (P * N + kQ * P) * 2 + (size_t)4 * (3 * kQ + 32) * sizeof(float) + (size_t)4 * 8 * P * sizeof(float);
+}
+
+template <typename T, int P, int N>
+__global__ void __launch_bounds__(256, (y16_smem<P, N>() <= 80 * 1024 ? 2 : 1))
+ssd_y16_kernel(const DiagArgs a) {
+    static_assert(sizeof(T) == 2, "16-bit operands only");
+    constexpr int BN = P / 32, KSN = N / 16;
+    constexpr int SPR_S = N / 8, SPR_X = P / 8;            // 16-byte slots per row
+    constexpr int NS = P * SPR_S / 256, NX = kQ * SPR_X / 256;   // direct-to-LDS loads per lane per tile
+    constexpr int TAB = 3 * kQ + 32;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* sS = reinterpret_cast<T*>(smem_raw);                       // [2][P][N]     swizzled slots
+    T* sX = sS + 2 * P * N;                                       // [2][kQ][P]    swizzled slots
+    float* wt_all = reinterpret_cast<float*>(sX + 2 * kQ * P);    // [4 waves][wl kQ | wd kQ | wv kQ | wu 32]
+    float* sY = wt_all + 4 * TAB;                                 // [4 waves][8][P]
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 31, half = lane >> 5;
+    const int64_t c = blockIdx.x, b = blockIdx.z;
+    const int64_t g = blockIdx.y / a.nslices, slice = blockIdx.y % a.nslices;
+    const int64_t hpg = a.nheads / a.ngroups;
+    const int64_t t0 = c * kQ;
+    const int valid = (int)((a.seqlen - t0) < kQ ? (a.seqlen - t0) : kQ);
+    const int row0 = wave * 32;
+    float* wl = wt_all + wave * TAB;
+    float* wd = wl + kQ;
+    float* wv = wd + kQ;
+    float* wu = wv + kQ;          // [32]: rows row0 .. row0 + 31
+    float* sYw = sY + wave * 8 * P;
+
+    // ---- asynchronous tile copy of one head into buffer `buf`
+    auto issue_tiles = [&](int64_t h, int buf) {
+        const T* Sp = static_cast<const T*>(a.S) + ((b * a.nchunks + c) * a.nheads + h) * (int64_t)(P * N);
+        T* dS = sS + buf * (P * N);
+#pragma unroll
+        for (int it = 0; it < NS; ++it) {
+            const int s0 = (wave * NS + it) * 64;              // first slot of this wave-wide load
+            const int s = s0 + lane;
+            const int row = s / SPR_S, cs = (s % SPR_S) ^ swz_s<SPR_S>(row);
+            async_copy16(Sp + row * N + cs * 8, dS + s0 * 8);
+        }
+        const T* Xp = static_cast<const T*>(a.Z) + b * a.Z_sb + t0 * a.Z_sl + h * a.Z_sh;
+        T* dX = sX + buf * (kQ * P);
+#pragma unroll
+        for (int it = 0; it < NX; ++it) {
+            const int s0 = (wave * NX + it) * 64;
+            const int s = s0 + lane;
+            const int row = s / SPR_X, cs = (s % SPR_X) ^ swz_x(row);
+            // rows past the end of the sequence re-read the last valid row: their dt is 0, so they only ever meet zeros
+            const int grow = row < valid ? row : valid - 1;
+            async_copy16(Xp + (int64_t)grow * a.Z_sl + cs * 8, dX + s0 * 8);
+        }
+    };
+
+    const int64_t h_first = g * hpg + slice * a.hps;
+    uint32_t pr0, pr1;            // raw dt of the head after the current one
+    wave_dt_load_raw<T>(a.dt, a.dt_f32, b * a.dt_sb + t0 * a.dt_sl + h_first, a.dt_sl, valid, pr0, pr1);
+    issue_tiles(h_first, 0);
+
+    // ---- head-independent operands, resident in registers
+    Frag<T> fd[8], fo[KSN];
+    {
+        const T* Gp = static_cast<const T*>(a.Gd) + ((b * a.nchunks + c) * a.ngroups + g) * (int64_t)(kQ * kQ) + (row0 + r) * kQ;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks)
+            if (ks <= 2 * wave + 1) fd[ks] = load_frag(Gp + ks * 16 + half * 8);
+        const T* Cp = static_cast<const T*>(a.Aoff) + b * a.Ao_sb + (t0 + row0 + r) * a.Ao_sl + g * a.Ao_sg;
+        const bool c_ok = row0 + r < valid;
+#pragma unroll
+        for (int ks = 0; ks < KSN; ++ks) {
+            if (c_ok) fo[ks] = load_frag(Cp + ks * 16 + half * 8);
+            else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) fo[ks].v[e] = (T)0.f;
+            }
+        }
+    }
+
+    for (int64_t hh = 0; hh < a.hps; ++hh) {
+        const int64_t h = h_first + hh;
+        const int buf = (int)(hh & 1);
+        const float Ah = a.A[h];
+        const float Dh = a.D ? a.D[h] : 0.f;
+
+        // ---- wave-private cumulative sum and decay tables
+        float d0, d1, l0, l1;
+        wave_dt_cvt<T>(a.dt_f32, valid, pr0, pr1, d0, d1);
+        wave_cumsum_from(Ah, d0, d1, l0, l1);
+        const float l_first = wave < 2 ? __shfl(l0, row0, 64) : __shfl(l1, row0 - 64, 64);
+        const float l_last = wave < 2 ? __shfl(l0, row0 + 31, 64) : __shfl(l1, row0 + 31 - 64, 64);
+        const bool fast = (l_first - l_last) < kMaxRange;
+        const float lref = l_first;
+        wl[lane] = l0; wl[lane + 64] = l1; wd[lane] = d0; wd[lane + 64] = d1;
+        wv[lane] = lane < row0 + 32 ? __expf(lref - l0) * d0 : 0.f;
+        wv[lane + 64] = lane + 64 < row0 + 32 ? __expf(lref - l1) * d1 : 0.f;
+        {
+            const float lmine = wave < 2 ? l0 : l1;                 // token row0 + (lane & 31) lives in lane (row0 & 63) + ...
+            const float lr = __shfl(lmine, (row0 & 63) + r, 64);
+            if (lane < 32) wu[lane] = __expf(fminf(lr - lref, 0.f));
+        }
+
+        wait_vmem_all();          // this wave's share of the tiles of head hh has landed
+        __syncthreads();          // ... and everyone's; every wave is also done with head hh-1 (the other buffer)
+        if (hh + 1 < a.hps) {
+            wave_dt_load_raw<T>(a.dt, a.dt_f32, b * a.dt_sb + t0 * a.dt_sl + h + 1, a.dt_sl, valid, pr0, pr1);
+            issue_tiles(h + 1, buf ^ 1);
+        }
+        const T* cS = sS + buf * (P * N);
+        const T* cX = sX + buf * (kQ * P);
+
+        const float off_fast = __expf(lref);
+        auto off_scale = [&](int v) -> float { return fast ? off_fast : __expf(wl[row0 + acc_row(lane, v)]); };
+        auto fin_scale = [&](int v) -> float { return fast ? wu[acc_row(lane, v)] : 1.f; };
+
+        // ---- off-diagonal term: C rows (registers) x S_prev (LDS, natural layout)
+        floatx16 acc[1][BN];
+        acc_zero(acc);
+#pragma unroll
+        for (int ks = 0; ks < KSN; ++ks) {
+#pragma unroll
+            for (int j = 0; j < BN; ++j) {
+                const int row = j * 32 + r;
+                const Frag<T> bf = load_frag(cS + (row * SPR_S + ((ks * 2 + half) ^ swz_s<SPR_S>(row))) * 8);
+                mma_frag(acc[0][j], fo[ks], bf);
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const float os = off_scale(v);
+#pragma unroll
+            for (int j = 0; j < BN; ++j) acc[0][j][v] *= os;
+        }
+
+        // ---- diagonal term: causal C B^T fragment scaled by the decay table along k; x through transpose reads
+        const int jrow = row0 + r;
+        const float l_row = wl[jrow];
+        // transpose read: the 16 lanes of a group fetch a [4 tokens][16 channels] block; lane (i0 = bits 3:2, i1 = bits 1:0)
+        // supplies the address of token i0, channels 4 i1 .. 4 i1 + 3 and receives channel (lane & 15) of tokens 0..3
+        const int tr_tok = 8 * half + ((lane >> 2) & 3);
+        const int tr_col = ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            if (ks > 2 * wave + 1) continue;
+            float f[8];
+            if (fast) {
+                const floatx4 fa = *reinterpret_cast<const floatx4*>(wv + ks * 16 + half * 8);
+                const floatx4 fb = *reinterpret_cast<const floatx4*>(wv + ks * 16 + half * 8 + 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { f[e] = fa[e]; f[4 + e] = fb[e]; }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int k = ks * 16 + half * 8 + e;
+                    f[e] = (k <= jrow) ? __expf(l_row - wl[k]) * wd[k] : 0.f;
+                }
+            }
+            const Frag<T> af = scale_frag(fd[ks], f);
+#pragma unroll
+            for (int j = 0; j < BN; ++j) {
+                const int col = j * 32 + tr_col;
+                const int ta = ks * 16 + tr_tok, tb = ta + 4;
+                typedef T tvec4 __attribute__((ext_vector_type(4)));
+                const tvec4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                    (M2_LDS tvec4*)(cX + (ta * SPR_X + ((col >> 3) ^ swz_x(ta))) * 8 + (col & 7)));
+                const tvec4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                    (M2_LDS tvec4*)(cX + (tb * SPR_X + ((col >> 3) ^ swz_x(tb))) * 8 + (col & 7)));
+                Frag<T> bf;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { bf.v[e] = lo[e]; bf.v[4 + e] = hi[e]; }
+                mma_frag(acc[0][j], af, bf);
+            }
+        }
+
+        // ---- epilogue, 8 token rows at a time: fp32 through the wave-private tile, then row-contiguous 16-byte
+        //      stores of  y = u * acc + D x  (x from the same LDS tile, row-wise)
+        constexpr int LPR = P / 8;               // lanes per output row
+        constexpr int RPP = 64 / LPR;            // rows per store pass
+        T* Yp = static_cast<T*>(a.Y) + b * a.Y_sb + t0 * a.Y_sl + h * a.Y_sh;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+#pragma unroll
+            for (int j = 0; j < BN; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sYw[(4 * half + e) * P + j * 32 + r] = acc[0][j][4 * q + e] * fin_scale(4 * q + e);
+            wave_lds_sync();
+#pragma unroll
+            for (int ps = 0; ps < 8 / RPP; ++ps) {
+                const int rl = ps * RPP + lane / LPR, cv = lane % LPR;
+                const int tok = row0 + 8 * q + rl;
+                const floatx4 ya = *reinterpret_cast<const floatx4*>(sYw + rl * P + cv * 8);
+                const floatx4 yb = *reinterpret_cast<const floatx4*>(sYw + rl * P + cv * 8 + 4);
+                const uint4 xr = *reinterpret_cast<const uint4*>(cX + (tok * SPR_X + (cv ^ swz_x(tok))) * 8);
+                const T* xe = reinterpret_cast<const T*>(&xr);
+                uint4 o;
+                T* oe = reinterpret_cast<T*>(&o);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    oe[e] = from_f32<T>(ya[e] + Dh * to_f32(xe[e]));
+                    oe[4 + e] = from_f32<T>(yb[e] + Dh * to_f32(xe[4 + e]));
+                }
+                if (tok < valid) *reinterpret_cast<uint4*>(Yp + (int64_t)tok * a.Y_sl + cv * 8) = o;
+            }
+            wave_lds_sync();
+        }
+    }
+}
+
+}  // namespace m2
