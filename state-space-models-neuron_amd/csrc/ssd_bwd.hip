@@ -518,10 +518,24 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         a.dX = p->dx; a.dX_sb = p->dx_stride_b; a.dX_sl = p->dx_stride_l; a.dX_sh = p->dx_stride_h;
         a.ddt = p->ddt; a.ddt_sb = p->ddt_stride_b; a.ddt_sl = p->ddt_stride_l;
         a.dl_diag = w.dl; a.dl_c = w.dlc; a.dlam = w.dlam; a.dAp = w.dAp; a.dDp = w.dDp;
-        auto k = diag_off_kernel<T, P, N, true>;
-        const size_t sm = diag_smem<T, P, N, true>();
-        if ((rc = allow_smem(k, sm))) return rc;
-        k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * a.nslices), (unsigned)p->batch), 256, sm, st>>>(a);
+        const dim3 grid((unsigned)nc, (unsigned)(p->ngroups * a.nslices), (unsigned)p->batch);
+        if constexpr (dx16_ok<T, P, N>()) {
+            auto k = ssd_dx16_kernel<T, P, N>;
+            const size_t sm = dx16_smem<P, N>();
+            if ((rc = allow_smem(k, sm))) return rc;
+            const Dx16Out o{w.dirp, w.rbp, w.dDp8};
+            k<<<grid, 512, sm, st>>>(a, o);
+            if ((rc = check_launch("ssd_dx16_kernel"))) return rc;
+            da_kernel<T><<<(unsigned)(p->batch * p->nheads * nc), 64, 0, st>>>(
+                p->dt, dt_f32, p->dt_stride_b, p->dt_stride_l, p->A, w.dl, w.dlc, w.dlam, w.dirp, w.rbp, w.dDp8,
+                p->ddt, p->ddt_stride_b, p->ddt_stride_l, w.dAp, w.dDp, p->seqlen, p->nheads, nc);
+            if ((rc = check_launch("ssd da_kernel"))) return rc;
+        } else {
+            auto k = diag_off_kernel<T, P, N, true>;
+            const size_t sm = diag_smem<T, P, N, true>();
+            if ((rc = allow_smem(k, sm))) return rc;
+            k<<<grid, 256, sm, st>>>(a);
+        }
         if ((rc = check_launch("ssd diag_off_kernel<bwd>"))) return rc;
     }
     {

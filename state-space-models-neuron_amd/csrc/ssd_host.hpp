@@ -2,6 +2,7 @@
 #pragma once
 #include "ssd_kernels.hpp"
 #include "ssd_diag.hpp"
+#include "ssd_dx.hpp"
 
 namespace m2 {
 
@@ -15,6 +16,7 @@ struct SsdWorkspace {
     void* dprev = nullptr; float* dlam = nullptr;
     float* dAp = nullptr; float* dDp = nullptr; float* dBp = nullptr; float* dCp = nullptr; float* dl = nullptr; float* dlc = nullptr; float* dGp = nullptr;
     float* dGs = nullptr; float* dBs = nullptr; float* dCs = nullptr;   // partials summed over the head slices
+    float* dirp = nullptr; float* rbp = nullptr; float* dDp8 = nullptr; // per channel-half / per-wave partials of the dx kernel
     int64_t nslices = 1, heads_per_slice = 1;
     size_t bytes = 0;
 };
@@ -79,6 +81,9 @@ inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd) {
         w.dDp = reinterpret_cast<float*>(take(bhc * 4));
         w.dl = reinterpret_cast<float*>(take(bhc * kQ * 4));
         w.dlc = reinterpret_cast<float*>(take(bhc * kQ * 4));
+        w.dirp = reinterpret_cast<float*>(take(bhc * 2 * kQ * 4));
+        w.rbp = reinterpret_cast<float*>(take(bhc * 2 * kQ * 4));
+        w.dDp8 = reinterpret_cast<float*>(take(bhc * 8 * 4));
         w.dGp = reinterpret_cast<float*>(take((size_t)p->batch * nc * p->ngroups * w.nslices * kQ * kQ * 4));
         const size_t part = (size_t)p->batch * nc * p->ngroups * w.nslices * kQ * p->dstate * 4;
         w.dBp = reinterpret_cast<float*>(take(part));
