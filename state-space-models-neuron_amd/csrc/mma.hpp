@@ -274,6 +274,15 @@ __device__ __forceinline__ void wave_chunk_cumsum(const void* __restrict__ dt, i
     wave_cumsum_from(A, d0, d1, l0, l1);
 }
 
+// Per (batch, head, chunk) the cumulative log-decay and dt are computed once (ld_table_kernel) into a table of
+// 2 * kQ floats, [ l[0..kQ) | dt[0..kQ) ], tokens past the end of the sequence holding dt = 0 and the last l.
+// Lane holds tokens `lane` and `lane + 64`.
+__device__ __forceinline__ void wave_ld_load(const float* __restrict__ ldtab, int64_t bhc, float& l0, float& l1, float& d0, float& d1) {
+    const int lane = threadIdx.x & 63;
+    const float* p = ldtab + bhc * (2 * kQ);
+    l0 = p[lane]; l1 = p[lane + 64]; d0 = p[kQ + lane]; d1 = p[kQ + lane + 64];
+}
+
 // Orders this wave's LDS writes before its later LDS reads of what OTHER lanes of the same wave wrote
 // (wave-private staging buffers).  The hardware executes one wave's LDS operations in order; the fences
 // keep the compiler from reordering them.

@@ -48,10 +48,10 @@ constexpr bool dg_g_in_lds() { return (size_t)14 * kQ * sizeof(float) + ((size_t
 
 template <typename T, int P>
 __global__ void __launch_bounds__(512, 2)
-dg_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f32, const float* __restrict__ A,
+dg_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
           const T* __restrict__ dY, const T* __restrict__ Gm, float* __restrict__ dGp, float* __restrict__ dl_diag,
           int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks, int64_t nslices, int64_t hps,
-          int64_t Xsb, int64_t Xsl, int64_t Xsh, int64_t dtsb, int64_t dtsl, int64_t dYsb, int64_t dYsl, int64_t dYsh) {
+          int64_t Xsb, int64_t Xsl, int64_t Xsh, int64_t dYsb, int64_t dYsl, int64_t dYsh) {
     constexpr int LDP = lds_ld<T>(P);
     constexpr int LDQ = lds_ld<T>(kQ);
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -102,7 +102,7 @@ dg_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f32, cons
     for (int64_t hh = 0; hh < hps; ++hh) {
         const int64_t h = g * hpg + slice * hps + hh;
         float l0, l1, d0, d1;
-        wave_chunk_cumsum<T>(dt, dt_f32, b * dtsb + t0 * dtsl + h, dtsl, valid, A[h], l0, l1, d0, d1);
+        wave_ld_load(ldtab, (b * nheads + h) * nchunks + c, l0, l1, d0, d1);
         wl[lane] = l0; wl[lane + 64] = l1;
         const float l_first = rb < 2 ? __shfl(l0, rb * 32, 64) : __shfl(l1, rb * 32 - 64, 64);
         const float l_last = rb < 2 ? __shfl(l0, rb * 32 + 31, 64) : __shfl(l1, rb * 32 + 31 - 64, 64);
@@ -191,12 +191,11 @@ constexpr bool off_c_in_lds() { return (size_t)10 * kQ * sizeof(float) + ((size_
 template <typename T, int P, int N, bool SIDE_C>
 __global__ void __launch_bounds__(512, SIDE_C ? 2 : 4)
 off_kernel(const T* __restrict__ Arow, int64_t Asb, int64_t Asl, int64_t Ash,      // dY (C side) or X (B side)
-           const void* __restrict__ dt, int dt_f32, const float* __restrict__ A,
+           const float* __restrict__ ldtab,
            const T* __restrict__ St,                                               // S_prev (C side) or dS (B side): [b][c][h][P][N]
            const T* __restrict__ Cm, int64_t Csb, int64_t Csl, int64_t Csg,        // C side only
            float* __restrict__ outp, float* __restrict__ dl_c,
-           int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks, int64_t nslices, int64_t hps,
-           int64_t dtsb, int64_t dtsl) {
+           int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks, int64_t nslices, int64_t hps) {
     constexpr int LDP = lds_ld<T>(P);
     constexpr int NB = N / 64;
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -250,7 +249,7 @@ off_kernel(const T* __restrict__ Arow, int64_t Asb, int64_t Asl, int64_t Ash,   
     for (int64_t hh = 0; hh < hps; ++hh) {
         const int64_t h = g * hpg + slice * hps + hh;
         float l0, l1, d0, d1;
-        wave_chunk_cumsum<T>(dt, dt_f32, b * dtsb + t0 * dtsl + h, dtsl, valid, A[h], l0, l1, d0, d1);
+        wave_ld_load(ldtab, (b * nheads + h) * nchunks + c, l0, l1, d0, d1);
         if (SIDE_C) { ws[lane] = __expf(l0); ws[lane + 64] = __expf(l1); }
         else {
             const float Lam = __shfl(l1, 63, 64);
@@ -470,8 +469,8 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         int64_t ns, hps;
         ssd_head_slicing(p, 1024, &ns, &hps);
         k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * ns), (unsigned)p->batch), 256, sm, st>>>(
-            dy, p->dt, dt_f32, p->A, static_cast<const T*>(w.Ct), w.local, w.lam, p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
-            p->dy_stride_b, p->dy_stride_l, p->dy_stride_h, p->dt_stride_b, p->dt_stride_l);
+            dy, w.ldtab, static_cast<const T*>(w.Ct), w.local, p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
+            p->dy_stride_b, p->dy_stride_l, p->dy_stride_h);
         if ((rc = check_launch("ssd chunk_state_kernel<dstate>"))) return rc;
         state_scan_kernel<T, P * N, true><<<dim3((unsigned)p->nheads, (unsigned)p->batch, kScanSplit), 256, 0, st>>>(
             w.local, w.lam, p->d_final_state, static_cast<T*>(w.dprev), p->d_initial_state,
@@ -479,13 +478,23 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         if ((rc = check_launch("ssd state_scan_kernel<reverse>"))) return rc;
     }
     {
-        auto k = dg_kernel<T, P>;
-        const size_t sm = dg_smem<T, P>();
-        if ((rc = allow_smem(k, sm))) return rc;
-        k<<<grid_s, 512, sm, st>>>(x, p->dt, dt_f32, p->A, dy, static_cast<const T*>(w.Gm), w.dGp, w.dl,
-                                   p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice,
-                                   p->x_stride_b, p->x_stride_l, p->x_stride_h, p->dt_stride_b, p->dt_stride_l,
-                                   p->dy_stride_b, p->dy_stride_l, p->dy_stride_h);
+        if constexpr (sizeof(T) == 2 && dg16_smem<P>() <= 160 * 1024) {
+            auto k = dg16_kernel<T, P>;
+            const size_t sm = dg16_smem<P>();
+            if ((rc = allow_smem(k, sm))) return rc;
+            k<<<grid_s, 512, sm, st>>>(x, w.ldtab, dy, w.G, w.dGp, w.dl,
+                                       p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice,
+                                       p->x_stride_b, p->x_stride_l, p->x_stride_h,
+                                       p->dy_stride_b, p->dy_stride_l, p->dy_stride_h);
+        } else {
+            auto k = dg_kernel<T, P>;
+            const size_t sm = dg_smem<T, P>();
+            if ((rc = allow_smem(k, sm))) return rc;
+            k<<<grid_s, 512, sm, st>>>(x, w.ldtab, dy, static_cast<const T*>(w.Gm), w.dGp, w.dl,
+                                       p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice,
+                                       p->x_stride_b, p->x_stride_l, p->x_stride_h,
+                                       p->dy_stride_b, p->dy_stride_l, p->dy_stride_h);
+        }
         if ((rc = check_launch("ssd dg_kernel"))) return rc;
     }
     {
@@ -494,15 +503,13 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         const size_t smc = off_smem<T, P, N>(true), sm = off_smem<T, P, N>(false);
         if ((rc = allow_smem(kc, smc))) return rc;
         if ((rc = allow_smem(kb, sm))) return rc;
-        kc<<<grid_s, 512, smc, st>>>(dy, p->dy_stride_b, p->dy_stride_l, p->dy_stride_h, p->dt, dt_f32, p->A,
+        kc<<<grid_s, 512, smc, st>>>(dy, p->dy_stride_b, p->dy_stride_l, p->dy_stride_h, w.ldtab,
                                     static_cast<const T*>(w.prev), Cm, p->C_stride_b, p->C_stride_l, p->C_stride_g,
-                                    w.dCp, w.dlc, p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice,
-                                    p->dt_stride_b, p->dt_stride_l);
+                                    w.dCp, w.dlc, p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice);
         if ((rc = check_launch("ssd off_kernel<C>"))) return rc;
-        kb<<<grid_s, 512, sm, st>>>(x, p->x_stride_b, p->x_stride_l, p->x_stride_h, p->dt, dt_f32, p->A,
+        kb<<<grid_s, 512, sm, st>>>(x, p->x_stride_b, p->x_stride_l, p->x_stride_h, w.ldtab,
                                     static_cast<const T*>(w.dprev), nullptr, 0, 0, 0,
-                                    w.dBp, nullptr, p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice,
-                                    p->dt_stride_b, p->dt_stride_l);
+                                    w.dBp, nullptr, p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice);
         if ((rc = check_launch("ssd off_kernel<B>"))) return rc;
     }
     {
@@ -517,6 +524,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         a.X = p->x; a.X_sb = p->x_stride_b; a.X_sl = p->x_stride_l; a.X_sh = p->x_stride_h;
         a.dX = p->dx; a.dX_sb = p->dx_stride_b; a.dX_sl = p->dx_stride_l; a.dX_sh = p->dx_stride_h;
         a.ddt = p->ddt; a.ddt_sb = p->ddt_stride_b; a.ddt_sl = p->ddt_stride_l;
+        a.ldtab = w.ldtab;
         a.dl_diag = w.dl; a.dl_c = w.dlc; a.dlam = w.dlam; a.dAp = w.dAp; a.dDp = w.dDp;
         const dim3 grid((unsigned)nc, (unsigned)(p->ngroups * a.nslices), (unsigned)p->batch);
         if constexpr (dx16_ok<T, P, N>()) {

@@ -29,6 +29,7 @@ constexpr float kMaxRange = 80.f;
 struct DiagArgs {
     // common
     const void* dt; int dt_f32; const float* A; const float* D;
+    const float* ldtab;         // [b][h][c][ l kQ | dt kQ ]
     const void* Aoff;           // C (fwd) or B (bwd): [b][l][g][N]
     int64_t Ao_sb, Ao_sl, Ao_sg;
     const void* Gd;             // masked CB^T (fwd) or its transpose (bwd): [b][c][g][kQ][kQ]
@@ -109,7 +110,7 @@ diag_off_kernel(const DiagArgs a) {
 
         // ---- wave-private cumulative sum and decay tables
         float l0, l1, d0, d1;
-        wave_chunk_cumsum<T>(a.dt, a.dt_f32, b * a.dt_sb + t0 * a.dt_sl + h, a.dt_sl, valid, Ah, l0, l1, d0, d1);
+        wave_ld_load(a.ldtab, (b * a.nheads + h) * a.nchunks + c, l0, l1, d0, d1);
         // l at the first / last token of this wave's row block (tokens 32w, 32w+31) and at the chunk end
         const float l_first = wave < 2 ? __shfl(l0, row0, 64) : __shfl(l1, row0 - 64, 64);
         const float l_last = wave < 2 ? __shfl(l0, row0 + 31, 64) : __shfl(l1, row0 + 31 - 64, 64);

@@ -22,7 +22,7 @@ namespace m2 {
 
 template <int P, int N>
 constexpr size_t dx16_smem() {
-    return (size_t)2 * (P * N + 2 * kQ * P) * 2 + (size_t)8 * (3 * kQ + 32) * sizeof(float) + (size_t)8 * 16 * (P / 2) * sizeof(float);
+    return (size_t)2 * ((P * N + 2 * kQ * P) * 2 + 2 * kQ * sizeof(float)) + (size_t)8 * (kQ + 32) * sizeof(float) + (size_t)8 * 16 * (P / 2) * sizeof(float);
 }
 template <typename T, int P, int N>
 constexpr bool dx16_ok() { return sizeof(T) == 2 && dx16_smem<P, N>() <= 160 * 1024; }
@@ -41,11 +41,12 @@ ssd_dx16_kernel(const DiagArgs a, const Dx16Out o) {
     constexpr int BN = PW / 32, KSN = N / 16;
     constexpr int SPR_S = N / 8, SPR_X = P / 8;
     constexpr int NS = P * SPR_S / 512, NX = kQ * SPR_X / 512;
-    constexpr int TAB = 3 * kQ + 32;
+    constexpr int TAB = kQ + 32;
     constexpr int TILES = P * N + 2 * kQ * P;    // elements per buffer
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* tiles = reinterpret_cast<T*>(smem_raw);                       // [2][ dS | dy | x ]
-    float* wt_all = reinterpret_cast<float*>(tiles + 2 * TILES);     // [8 waves][wl kQ | wd kQ | wv kQ | wu 32]
+    float* sLD = reinterpret_cast<float*>(tiles + 2 * TILES);        // [2][ l kQ | dt kQ ]
+    float* wt_all = sLD + 2 * 2 * kQ;                                // [8 waves][wv kQ | wu 32]
     float* sY = wt_all + 8 * TAB;                                    // [8 waves][16][PW]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -57,9 +58,7 @@ ssd_dx16_kernel(const DiagArgs a, const Dx16Out o) {
     const int64_t t0 = c * kQ;
     const int valid = (int)((a.seqlen - t0) < kQ ? (a.seqlen - t0) : kQ);
     const int row0 = rbk * 32, col0 = ch * PW;
-    float* wl = wt_all + wave * TAB;
-    float* wd = wl + kQ;
-    float* wv = wd + kQ;
+    float* wv = wt_all + wave * TAB;
     float* wu = wv + kQ;
     float* sYw = sY + wave * 16 * PW;
 
@@ -84,11 +83,10 @@ ssd_dx16_kernel(const DiagArgs a, const Dx16Out o) {
             async_copy16(Yp + (int64_t)grow * a.Z_sl + cs * 8, dY + s0 * 8);
             async_copy16(Xp + (int64_t)grow * a.X_sl + cs * 8, dXt + s0 * 8);
         }
+        async_copy_ldtab(a.ldtab, (b * a.nheads + h) * a.nchunks + c, sLD + buf * 2 * kQ);
     };
 
     const int64_t h_first = g * hpg + slice * a.hps;
-    uint32_t pr0, pr1;
-    wave_dt_load_raw<T>(a.dt, a.dt_f32, b * a.dt_sb + t0 * a.dt_sl + h_first, a.dt_sl, valid, pr0, pr1);
     issue_tiles(h_first, 0);
 
     // ---- head-independent operands, resident in registers: B rows and (causal C B^T)^T rows of this wave's tokens
@@ -118,39 +116,26 @@ ssd_dx16_kernel(const DiagArgs a, const Dx16Out o) {
         const int64_t h = h_first + hh;
         const int buf = (int)(hh & 1);
         const int64_t bhc = (b * a.nheads + h) * a.nchunks + c;
-        const float Ah = a.A[h];
         const float Dh = a.D ? a.D[h] : 0.f;
 
-        // ---- wave-private cumulative sum and decay tables
-        float d0, d1, l0, l1;
-        wave_dt_cvt<T>(a.dt_f32, valid, pr0, pr1, d0, d1);
-        wave_cumsum_from(Ah, d0, d1, l0, l1);
-        const float l_first = rbk < 2 ? __shfl(l0, row0, 64) : __shfl(l1, row0 - 64, 64);
-        const float l_last = rbk < 2 ? __shfl(l0, row0 + 31, 64) : __shfl(l1, row0 + 31 - 64, 64);
-        const float Lam = __shfl(l1, 63, 64);
+        wait_vmem_all();          // this wave's share of the tiles of head hh, and the whole [ l | dt ] table, have landed
+        // ---- wave-private decay tables from the shared [ l | dt ] table
+        const float* sl = sLD + buf * 2 * kQ;
+        const float* sd = sl + kQ;
+        const float l_first = sl[row0], l_last = sl[row0 + 31], Lam = sl[kQ - 1];
         const bool fast = (l_first - l_last) < kMaxRange;
         const float lref = l_last;
-        wl[lane] = l0; wl[lane + 64] = l1; wd[lane] = d0; wd[lane + 64] = d1;
-        wv[lane] = lane >= row0 ? __expf(l0 - lref) : 0.f;
-        wv[lane + 64] = lane + 64 >= row0 ? __expf(l1 - lref) : 0.f;
-        {
-            const float lmine = rbk < 2 ? l0 : l1;
-            const float lr = __shfl(lmine, (row0 & 63) + r, 64);
-            if (lane < 32) wu[lane] = __expf(fminf(lref - lr, 0.f));
-        }
-
-        wait_vmem_all();
+        wv[lane] = lane >= row0 ? __expf(sl[lane] - lref) : 0.f;
+        wv[lane + 64] = lane + 64 >= row0 ? __expf(sl[lane + 64] - lref) : 0.f;
+        if (lane < 32) wu[lane] = __expf(fminf(lref - sl[row0 + lane], 0.f));
         __syncthreads();
-        if (hh + 1 < a.hps) {
-            wave_dt_load_raw<T>(a.dt, a.dt_f32, b * a.dt_sb + t0 * a.dt_sl + h + 1, a.dt_sl, valid, pr0, pr1);
-            issue_tiles(h + 1, buf ^ 1);
-        }
+        if (hh + 1 < a.hps) issue_tiles(h + 1, buf ^ 1);
         const T* cS = tiles + buf * TILES;
         const T* cY = cS + P * N;
         const T* cX = cY + kQ * P;
 
         const float off_fast = __expf(Lam - lref);
-        auto off_scale = [&](int v) -> float { return fast ? off_fast : __expf(Lam - wl[row0 + acc_row(lane, v)]); };
+        auto off_scale = [&](int v) -> float { return fast ? off_fast : __expf(Lam - sl[row0 + acc_row(lane, v)]); };
         auto fin_scale = [&](int v) -> float { return fast ? wu[acc_row(lane, v)] : 1.f; };
 
         // ---- off-diagonal term: B rows (registers) x dS (LDS, natural layout)
@@ -193,12 +178,12 @@ ssd_dx16_kernel(const DiagArgs a, const Dx16Out o) {
             int ri;
             const float tot = half_wave_reduce16(rbv, &ri);
             const int row = row0 + acc_row(lane, ri);
-            if ((lane & 1) == 0) o.rbp[(bhc * 2 + ch) * kQ + row] = tot * wd[row];
+            if ((lane & 1) == 0) o.rbp[(bhc * 2 + ch) * kQ + row] = tot * sd[row];
         }
 
         // ---- diagonal term: transposed causal C B^T fragment scaled along k = i; dy through transpose reads
         const int jrow = row0 + r;
-        const float l_row = wl[jrow];
+        const float l_row = sl[jrow];
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             if (ks < 2 * rbk) continue;
@@ -212,7 +197,7 @@ ssd_dx16_kernel(const DiagArgs a, const Dx16Out o) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const int k = ks * 16 + half * 8 + e;
-                    f[e] = (k >= jrow) ? __expf(wl[k] - l_row) : 0.f;
+                    f[e] = (k >= jrow) ? __expf(sl[k] - l_row) : 0.f;
                 }
             }
             const Frag<T> af = scale_frag(fd[ks], f);
@@ -260,7 +245,7 @@ ssd_dx16_kernel(const DiagArgs a, const Dx16Out o) {
                 const uint4 gr = *reinterpret_cast<const uint4*>(cY + (tok * SPR_X + slot) * 8);
                 const T* xe = reinterpret_cast<const T*>(&xr);
                 const T* ge = reinterpret_cast<const T*>(&gr);
-                const float dtt = wd[tok];
+                const float dtt = sd[tok];
                 uint4 ov;
                 T* oe = reinterpret_cast<T*>(&ov);
                 float dir = 0.f, dd = 0.f;

@@ -125,7 +125,7 @@ int ssd_fwd_impl(const m2_ssd_params* p, hipStream_t st) {
     DiagArgs a{};
     a.dt = p->dt; a.dt_f32 = p->dt_dtype == M2_F32; a.A = p->A; a.D = p->D;
     a.Aoff = p->C; a.Ao_sb = p->C_stride_b; a.Ao_sl = p->C_stride_l; a.Ao_sg = p->C_stride_g;
-    a.Gd = w.Gm; a.S = w.prev;
+    a.Gd = w.Gm; a.S = w.prev; a.ldtab = w.ldtab;
     a.Z = p->x; a.Z_sb = p->x_stride_b; a.Z_sl = p->x_stride_l; a.Z_sh = p->x_stride_h;
     a.dt_sb = p->dt_stride_b; a.dt_sl = p->dt_stride_l;
     a.seqlen = p->seqlen; a.nheads = p->nheads; a.ngroups = p->ngroups; a.nchunks = nc;

@@ -3,6 +3,7 @@
 #include "ssd_kernels.hpp"
 #include "ssd_diag.hpp"
 #include "ssd_dx.hpp"
+#include "ssd_dg.hpp"
 
 namespace m2 {
 
@@ -13,6 +14,7 @@ namespace m2 {
 struct SsdWorkspace {
     float* G = nullptr; float* local = nullptr; void* prev = nullptr; float* lam = nullptr;
     void* Gm = nullptr; void* Gmt = nullptr; void* Bt = nullptr; void* Ct = nullptr;
+    float* ldtab = nullptr;             // [b][h][c][ l kQ | dt kQ ]
     void* dprev = nullptr; float* dlam = nullptr;
     float* dAp = nullptr; float* dDp = nullptr; float* dBp = nullptr; float* dCp = nullptr; float* dl = nullptr; float* dlc = nullptr; float* dGp = nullptr;
     float* dGs = nullptr; float* dBs = nullptr; float* dCs = nullptr;   // partials summed over the head slices
@@ -68,6 +70,7 @@ inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd) {
     if (p->chunk_states) w.prev = p->chunk_states;      // caller keeps the chunk states (forward -> backward)
     else w.prev = take(tiles * esz);
     w.lam = reinterpret_cast<float*>(take(bhc * 4));
+    w.ldtab = reinterpret_cast<float*>(take(bhc * 2 * kQ * 4));
     const size_t grp = (size_t)p->batch * nc * p->ngroups;
     w.Gm = take(grp * kQ * kQ * esz);
     w.Gmt = take(grp * kQ * kQ * esz);
@@ -143,6 +146,12 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
     const int dt_f32 = p->dt_dtype == M2_F32;
     int rc;
     {
+        const int64_t total = p->batch * p->nheads * nc;
+        ld_table_kernel<T><<<(unsigned)ceil_div(total, (int64_t)4), 256, 0, st>>>(p->dt, dt_f32, p->A, w.ldtab, w.lam, p->seqlen, p->nheads, nc, total,
+                                                                                p->dt_stride_b, p->dt_stride_l);
+        if ((rc = check_launch("ssd ld_table_kernel"))) return rc;
+    }
+    {
         auto k = cb_kernel<T, N>;
         const size_t sm = cb_smem<T>();
         if ((rc = allow_smem(k, sm))) return rc;
@@ -160,8 +169,8 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
         ssd_head_slicing(p, 1024, &ns, &hps);
         M2_REQUIRE(p->ngroups * ns <= 65535, M2_ERR_SHAPE, "ssd: too many group slices");
         k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * ns), (unsigned)p->batch), 256, sm, st>>>(
-            x, p->dt, dt_f32, p->A, static_cast<const T*>(w.Bt), w.local, w.lam, p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
-            p->x_stride_b, p->x_stride_l, p->x_stride_h, p->dt_stride_b, p->dt_stride_l);
+            x, w.ldtab, static_cast<const T*>(w.Bt), w.local, p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
+            p->x_stride_b, p->x_stride_l, p->x_stride_h);
         if ((rc = check_launch("ssd chunk_state_kernel"))) return rc;
     }
     {

@@ -104,19 +104,40 @@ cb_kernel(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict_
 }
 
 // ------------------------------------------------------------------------------------------
+// Cumulative log-decay table: one wave per (batch, head, chunk); ldtab[bhc] = [ l[0..kQ) | dt[0..kQ) ] in fp32,
+// l = inclusive cumsum of A_h dt within the chunk, lam[bhc] = l[kQ-1].  Every other kernel reads this table instead
+// of gathering dt (stride = nheads elements) and scanning it again per head.
+template <typename T>
+__global__ void __launch_bounds__(256)
+ld_table_kernel(const void* __restrict__ dt, int dt_f32, const float* __restrict__ A, float* __restrict__ ldtab,
+                float* __restrict__ lam, int64_t seqlen, int64_t nheads, int64_t nchunks, int64_t total,
+                int64_t dtsb, int64_t dtsl) {
+    const int lane = threadIdx.x & 63;
+    const int64_t bhc = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (bhc >= total) return;
+    const int64_t c = bhc % nchunks, h = (bhc / nchunks) % nheads, b = bhc / (nchunks * nheads);
+    const int64_t t0 = c * kQ;
+    const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
+    float l0, l1, d0, d1;
+    wave_chunk_cumsum<T>(dt, dt_f32, b * dtsb + t0 * dtsl + h, dtsl, valid, A[h], l0, l1, d0, d1);
+    float* p = ldtab + bhc * (2 * kQ);
+    p[lane] = l0; p[lane + 64] = l1; p[kQ + lane] = d0; p[kQ + lane + 64] = d1;
+    if (lane == 63) lam[bhc] = l1;
+}
+
+// ------------------------------------------------------------------------------------------
 // Local chunk state.  grid (nchunks, ngroups * nslices, batch), 256 threads; a workgroup loops over `hps` heads.
 //   DSTATE == false:  out[p][n] = sum_j (dt_j e^{Lam-l_j}) x[j][p] * B[j][n]      (forward)
 //   DSTATE == true :  out[p][n] = sum_i e^{l_i} dy[i][p] * C[i][n]                (backward)
 // `X` is x or dy; `Mt` is the group's B or C tile already transposed to [N][kQ] (tokens contiguous) by cb_kernel,
 // staged into LDS once per workgroup.  Per head only the x tile moves: it is loaded 16 bytes at a time, scaled in
 // fp32 and written transposed; the next head's tile is prefetched into registers while the MFMAs run.
-// Also writes lam[b][h][c] = Lam.
 template <typename T, int P, int N, bool DSTATE>
 __global__ void __launch_bounds__(256)
-chunk_state_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f32, const float* __restrict__ A,
-                   const T* __restrict__ Mt, float* __restrict__ out, float* __restrict__ lam,
+chunk_state_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
+                   const T* __restrict__ Mt, float* __restrict__ out,
                    int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks, int64_t nslices, int64_t hps,
-                   int64_t Xsb, int64_t Xsl, int64_t Xsh, int64_t dtsb, int64_t dtsl) {
+                   int64_t Xsb, int64_t Xsl, int64_t Xsh) {
     constexpr int LD = lds_ld<T>(kQ);
     constexpr int V = VecTraits<T>::kVec;
     constexpr int NIT = (P / V) / 2;              // 16-byte vectors per thread per head (thread <-> fixed token)
@@ -147,7 +168,7 @@ chunk_state_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_
     for (int64_t hh = 0; hh < hps; ++hh) {
         const int64_t h = g * hpg + slice * hps + hh;
         float l0, l1, d0, d1;
-        wave_chunk_cumsum<T>(dt, dt_f32, b * dtsb + t0 * dtsl + h, dtsl, valid, A[h], l0, l1, d0, d1);
+        wave_ld_load(ldtab, (b * nheads + h) * nchunks + c, l0, l1, d0, d1);
         const float Lam = __shfl(l1, 63, 64);
         // scale of this thread's token (token = lane + 64 * (wave & 1))
         const float lt = (wave & 1) ? l1 : l0, dtt = (wave & 1) ? d1 : d0;
@@ -176,7 +197,6 @@ chunk_state_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_
                     const int col = wn * (N / 2) + j * 32 + acc_col(lane);
                     op[row * N + col] = acc[i][j][v];
                 }
-        if (tid == 0 && lam) lam[(b * nheads + h) * nchunks + c] = Lam;
     }
 }
 

@@ -30,7 +30,24 @@ namespace m2 {
 // wait until this wave's outstanding vector-memory operations (including direct-to-LDS loads) are done;
 // the export and LDS/scalar counters are left alone.  gfx9 encoding: vmcnt = simm16[15:14,3:0], expcnt [6:4],
 // lgkmcnt [11:8].
-__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+// A compiler-level memory fence follows, so that no read of the copied data is scheduled before the wait.
+__device__ __forceinline__ void wait_vmem_all() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    asm volatile("" ::: "memory");
+}
+// ... until at most `groups` * PER of them are still outstanding (vector-memory operations retire in issue order, so
+// this leaves the youngest ones in flight).  `groups` must be wave-uniform.  Operations the caller did not count
+// (the compiler's own loads and stores) only make the wait longer, never too short.
+template <int PER>
+__device__ __forceinline__ void wait_vmem_keep(int groups) {
+    static_assert(3 * PER < 64, "vmcnt is a 6-bit counter");
+    constexpr int n1 = PER, n2 = 2 * PER, n3 = 3 * PER;
+    if (groups <= 0) __builtin_amdgcn_s_waitcnt(0x0F70);
+    else if (groups == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (n1 & 0xF) | ((n1 >> 4) << 14));
+    else if (groups == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (n2 & 0xF) | ((n2 >> 4) << 14));
+    else __builtin_amdgcn_s_waitcnt(0x0F70 | (n3 & 0xF) | ((n3 >> 4) << 14));
+    asm volatile("" ::: "memory");
+}
 
 // Asynchronous 16-byte-per-lane copy global -> LDS: lane i's 16 bytes land at lds_base + 16 i (lds_base wave-uniform).
 // Written as inline assembly on purpose: for the compiler's own direct-to-LDS builtin the wait-count pass
@@ -43,13 +60,20 @@ __device__ __forceinline__ void async_copy16(const void* gsrc, void* lds_base) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gsrc), "s"(l) : "memory", "m0");
 }
 
+// The [ l | dt ] table of one (batch, head, chunk): 2 kQ floats = 64 lanes x 16 bytes, one wave-wide copy.  Every
+// wave of the workgroup issues it (same source, same destination, same data), so each wave may read the table as
+// soon as ITS OWN copies have landed, and all waves issue the same number of vector-memory operations per head.
+__device__ __forceinline__ void async_copy_ldtab(const float* __restrict__ ldtab, int64_t bhc, float* lds_tab) {
+    async_copy16(ldtab + bhc * (2 * kQ) + (threadIdx.x & 63) * 4, lds_tab);
+}
+
 // 16-byte slot s of row `row` lives at slot (s ^ swz) of that row
 template <int SPR> __device__ __forceinline__ int swz_s(int row) { return row & (SPR - 1); }          // S_prev tile
 __device__ __forceinline__ int swz_x(int row) { return ((row >> 1) & 1) << 2; }                      // x tile
 
 template <int P, int N>
 constexpr size_t y16_smem() {
-    return (size_t)2 * (P * N + kQ * P) * 2 + (size_t)4 * (3 * kQ + 32) * sizeof(float) + (size_t)4 * 8 * P * sizeof(float);
+    return (size_t)2 * ((P * N + kQ * P) * 2 + 2 * kQ * sizeof(float)) + (size_t)4 * (kQ + 32) * sizeof(float) + (size_t)4 * 8 * P * sizeof(float);
 }
 
 template <typename T, int P, int N>
@@ -59,11 +83,12 @@ ssd_y16_kernel(const DiagArgs a) {
     constexpr int BN = P / 32, KSN = N / 16;
     constexpr int SPR_S = N / 8, SPR_X = P / 8;            // 16-byte slots per row
     constexpr int NS = P * SPR_S / 256, NX = kQ * SPR_X / 256;   // direct-to-LDS loads per lane per tile
-    constexpr int TAB = 3 * kQ + 32;
+    constexpr int TAB = kQ + 32;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* sS = reinterpret_cast<T*>(smem_raw);                       // [2][P][N]     swizzled slots
     T* sX = sS + 2 * P * N;                                       // [2][kQ][P]    swizzled slots
-    float* wt_all = reinterpret_cast<float*>(sX + 2 * kQ * P);    // [4 waves][wl kQ | wd kQ | wv kQ | wu 32]
+    float* sLD = reinterpret_cast<float*>(sX + 2 * kQ * P);       // [2][ l kQ | dt kQ ]
+    float* wt_all = sLD + 2 * 2 * kQ;                             // [4 waves][wv kQ | wu 32]
     float* sY = wt_all + 4 * TAB;                                 // [4 waves][8][P]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -74,9 +99,7 @@ ssd_y16_kernel(const DiagArgs a) {
     const int64_t t0 = c * kQ;
     const int valid = (int)((a.seqlen - t0) < kQ ? (a.seqlen - t0) : kQ);
     const int row0 = wave * 32;
-    float* wl = wt_all + wave * TAB;
-    float* wd = wl + kQ;
-    float* wv = wd + kQ;
+    float* wv = wt_all + wave * TAB;
     float* wu = wv + kQ;          // [32]: rows row0 .. row0 + 31
     float* sYw = sY + wave * 8 * P;
 
@@ -102,11 +125,10 @@ ssd_y16_kernel(const DiagArgs a) {
             const int grow = row < valid ? row : valid - 1;
             async_copy16(Xp + (int64_t)grow * a.Z_sl + cs * 8, dX + s0 * 8);
         }
+        async_copy_ldtab(a.ldtab, (b * a.nheads + h) * a.nchunks + c, sLD + buf * 2 * kQ);
     };
 
     const int64_t h_first = g * hpg + slice * a.hps;
-    uint32_t pr0, pr1;            // raw dt of the head after the current one
-    wave_dt_load_raw<T>(a.dt, a.dt_f32, b * a.dt_sb + t0 * a.dt_sl + h_first, a.dt_sl, valid, pr0, pr1);
     issue_tiles(h_first, 0);
 
     // ---- head-independent operands, resident in registers
@@ -131,37 +153,25 @@ ssd_y16_kernel(const DiagArgs a) {
     for (int64_t hh = 0; hh < a.hps; ++hh) {
         const int64_t h = h_first + hh;
         const int buf = (int)(hh & 1);
-        const float Ah = a.A[h];
         const float Dh = a.D ? a.D[h] : 0.f;
 
-        // ---- wave-private cumulative sum and decay tables
-        float d0, d1, l0, l1;
-        wave_dt_cvt<T>(a.dt_f32, valid, pr0, pr1, d0, d1);
-        wave_cumsum_from(Ah, d0, d1, l0, l1);
-        const float l_first = wave < 2 ? __shfl(l0, row0, 64) : __shfl(l1, row0 - 64, 64);
-        const float l_last = wave < 2 ? __shfl(l0, row0 + 31, 64) : __shfl(l1, row0 + 31 - 64, 64);
+        wait_vmem_all();          // this wave's share of the tiles of head hh, and the whole [ l | dt ] table, have landed
+        // ---- wave-private decay tables from the shared [ l | dt ] table
+        const float* sl = sLD + buf * 2 * kQ;
+        const float* sd = sl + kQ;
+        const float l_first = sl[row0], l_last = sl[row0 + 31];
         const bool fast = (l_first - l_last) < kMaxRange;
         const float lref = l_first;
-        wl[lane] = l0; wl[lane + 64] = l1; wd[lane] = d0; wd[lane + 64] = d1;
-        wv[lane] = lane < row0 + 32 ? __expf(lref - l0) * d0 : 0.f;
-        wv[lane + 64] = lane + 64 < row0 + 32 ? __expf(lref - l1) * d1 : 0.f;
-        {
-            const float lmine = wave < 2 ? l0 : l1;                 // token row0 + (lane & 31) lives in lane (row0 & 63) + ...
-            const float lr = __shfl(lmine, (row0 & 63) + r, 64);
-            if (lane < 32) wu[lane] = __expf(fminf(lr - lref, 0.f));
-        }
-
-        wait_vmem_all();          // this wave's share of the tiles of head hh has landed
-        __syncthreads();          // ... and everyone's; every wave is also done with head hh-1 (the other buffer)
-        if (hh + 1 < a.hps) {
-            wave_dt_load_raw<T>(a.dt, a.dt_f32, b * a.dt_sb + t0 * a.dt_sl + h + 1, a.dt_sl, valid, pr0, pr1);
-            issue_tiles(h + 1, buf ^ 1);
-        }
+        wv[lane] = lane < row0 + 32 ? __expf(lref - sl[lane]) * sd[lane] : 0.f;
+        wv[lane + 64] = lane + 64 < row0 + 32 ? __expf(lref - sl[lane + 64]) * sd[lane + 64] : 0.f;
+        if (lane < 32) wu[lane] = __expf(fminf(sl[row0 + lane] - lref, 0.f));
+        __syncthreads();          // everyone's share has landed; every wave is also done with head hh-1 (the other buffer)
+        if (hh + 1 < a.hps) issue_tiles(h + 1, buf ^ 1);
         const T* cS = sS + buf * (P * N);
         const T* cX = sX + buf * (kQ * P);
 
         const float off_fast = __expf(lref);
-        auto off_scale = [&](int v) -> float { return fast ? off_fast : __expf(wl[row0 + acc_row(lane, v)]); };
+        auto off_scale = [&](int v) -> float { return fast ? off_fast : __expf(sl[row0 + acc_row(lane, v)]); };
         auto fin_scale = [&](int v) -> float { return fast ? wu[acc_row(lane, v)] : 1.f; };
 
         // ---- off-diagonal term: C rows (registers) x S_prev (LDS, natural layout)
@@ -185,7 +195,7 @@ ssd_y16_kernel(const DiagArgs a) {
 
         // ---- diagonal term: causal C B^T fragment scaled by the decay table along k; x through transpose reads
         const int jrow = row0 + r;
-        const float l_row = wl[jrow];
+        const float l_row = sl[jrow];
         // transpose read: the 16 lanes of a group fetch a [4 tokens][16 channels] block; lane (i0 = bits 3:2, i1 = bits 1:0)
         // supplies the address of token i0, channels 4 i1 .. 4 i1 + 3 and receives channel (lane & 15) of tokens 0..3
         const int tr_tok = 8 * half + ((lane >> 2) & 3);
@@ -203,7 +213,7 @@ ssd_y16_kernel(const DiagArgs a) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const int k = ks * 16 + half * 8 + e;
-                    f[e] = (k <= jrow) ? __expf(l_row - wl[k]) * wd[k] : 0.f;
+                    f[e] = (k <= jrow) ? __expf(l_row - sl[k]) * sd[k] : 0.f;
                 }
             }
             const Frag<T> af = scale_frag(fd[ks], f);
