@@ -456,8 +456,10 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
     const T* x = static_cast<const T*>(p->x);
     const T* Cm = static_cast<const T*>(p->C);
     const T* dy = static_cast<const T*>(p->dy);
-    const dim3 grid_s((unsigned)nc, (unsigned)(p->ngroups * w.nslices), (unsigned)p->batch);
-    M2_REQUIRE(p->ngroups * w.nslices <= 65535, M2_ERR_SHAPE, "ssd_bwd: too many group slices");
+    const dim3 grid_g((unsigned)nc, (unsigned)(p->ngroups * w.ns_g), (unsigned)p->batch);
+    const dim3 grid_c((unsigned)nc, (unsigned)(p->ngroups * w.ns_c), (unsigned)p->batch);
+    const dim3 grid_b((unsigned)nc, (unsigned)(p->ngroups * w.ns_b), (unsigned)p->batch);
+    M2_REQUIRE(p->nheads <= 65535, M2_ERR_SHAPE, "ssd_bwd: too many group slices");
     int rc;
     // G (+ operand tiles); the state entering each chunk, unless the caller kept the forward's
     if ((rc = ssd_launch_states<T, P, N>(p, w, nullptr, st, p->chunk_states != nullptr))) return rc;
@@ -467,7 +469,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         const size_t sm = state_smem<T, P, N>();
         if ((rc = allow_smem(k, sm))) return rc;
         int64_t ns, hps;
-        ssd_head_slicing(p, 1024, &ns, &hps);
+        ssd_slicing(p, kWgsChunkState, &ns, &hps);
         k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * ns), (unsigned)p->batch), 256, sm, st>>>(
             dy, w.ldtab, static_cast<const T*>(w.Ct), w.local, p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
             p->dy_stride_b, p->dy_stride_l, p->dy_stride_h);
@@ -482,16 +484,16 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
             auto k = dg16_kernel<T, P>;
             const size_t sm = dg16_smem<P>();
             if ((rc = allow_smem(k, sm))) return rc;
-            k<<<grid_s, 512, sm, st>>>(x, w.ldtab, dy, w.G, w.dGp, w.dl,
-                                       p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice,
+            k<<<grid_g, 512, sm, st>>>(x, w.ldtab, dy, w.G, w.dGp, w.dl,
+                                       p->seqlen, p->nheads, p->ngroups, nc, w.ns_g, w.hps_g,
                                        p->x_stride_b, p->x_stride_l, p->x_stride_h,
                                        p->dy_stride_b, p->dy_stride_l, p->dy_stride_h);
         } else {
             auto k = dg_kernel<T, P>;
             const size_t sm = dg_smem<T, P>();
             if ((rc = allow_smem(k, sm))) return rc;
-            k<<<grid_s, 512, sm, st>>>(x, w.ldtab, dy, static_cast<const T*>(w.Gm), w.dGp, w.dl,
-                                       p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice,
+            k<<<grid_g, 512, sm, st>>>(x, w.ldtab, dy, static_cast<const T*>(w.Gm), w.dGp, w.dl,
+                                       p->seqlen, p->nheads, p->ngroups, nc, w.ns_g, w.hps_g,
                                        p->x_stride_b, p->x_stride_l, p->x_stride_h,
                                        p->dy_stride_b, p->dy_stride_l, p->dy_stride_h);
         }
@@ -503,13 +505,13 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         const size_t smc = off_smem<T, P, N>(true), sm = off_smem<T, P, N>(false);
         if ((rc = allow_smem(kc, smc))) return rc;
         if ((rc = allow_smem(kb, sm))) return rc;
-        kc<<<grid_s, 512, smc, st>>>(dy, p->dy_stride_b, p->dy_stride_l, p->dy_stride_h, w.ldtab,
+        kc<<<grid_c, 512, smc, st>>>(dy, p->dy_stride_b, p->dy_stride_l, p->dy_stride_h, w.ldtab,
                                     static_cast<const T*>(w.prev), Cm, p->C_stride_b, p->C_stride_l, p->C_stride_g,
-                                    w.dCp, w.dlc, p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice);
+                                    w.dCp, w.dlc, p->seqlen, p->nheads, p->ngroups, nc, w.ns_c, w.hps_c);
         if ((rc = check_launch("ssd off_kernel<C>"))) return rc;
-        kb<<<grid_s, 512, sm, st>>>(x, p->x_stride_b, p->x_stride_l, p->x_stride_h, w.ldtab,
+        kb<<<grid_b, 512, sm, st>>>(x, p->x_stride_b, p->x_stride_l, p->x_stride_h, w.ldtab,
                                     static_cast<const T*>(w.dprev), nullptr, 0, 0, 0,
-                                    w.dBp, nullptr, p->seqlen, p->nheads, p->ngroups, nc, w.nslices, w.heads_per_slice);
+                                    w.dBp, nullptr, p->seqlen, p->nheads, p->ngroups, nc, w.ns_b, w.hps_b);
         if ((rc = check_launch("ssd off_kernel<B>"))) return rc;
     }
     {
@@ -520,7 +522,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         a.Z = p->dy; a.Z_sb = p->dy_stride_b; a.Z_sl = p->dy_stride_l; a.Z_sh = p->dy_stride_h;
         a.dt_sb = p->dt_stride_b; a.dt_sl = p->dt_stride_l;
         a.seqlen = p->seqlen; a.nheads = p->nheads; a.ngroups = p->ngroups; a.nchunks = nc;
-        ssd_head_slicing(p, 1024, &a.nslices, &a.hps);
+        ssd_slicing(p, dx16_ok<T, P, N>() ? kWgsDx : 2, &a.nslices, &a.hps);
         a.X = p->x; a.X_sb = p->x_stride_b; a.X_sl = p->x_stride_l; a.X_sh = p->x_stride_h;
         a.dX = p->dx; a.dX_sb = p->dx_stride_b; a.dX_sl = p->dx_stride_l; a.dX_sh = p->dx_stride_h;
         a.ddt = p->ddt; a.ddt_sb = p->ddt_stride_b; a.ddt_sl = p->ddt_stride_l;
@@ -552,13 +554,19 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         if ((rc = allow_smem(k, sm))) return rc;
         const int64_t ngrp = p->batch * nc * p->ngroups;
         const float *gs = w.dGp, *cs = w.dCp, *bs = w.dBp;
-        if (w.nslices > 1) {
-            slice_sum_kernel<<<(unsigned)ceil_div(ngrp * kQ * kQ / 4, (int64_t)256), 256, 0, st>>>(w.dGp, w.dGs, ngrp, w.nslices, (int64_t)kQ * kQ);
-            slice_sum_kernel<<<(unsigned)ceil_div(ngrp * kQ * N / 4, (int64_t)256), 256, 0, st>>>(w.dCp, w.dCs, ngrp, w.nslices, (int64_t)kQ * N);
-            slice_sum_kernel<<<(unsigned)ceil_div(ngrp * kQ * N / 4, (int64_t)256), 256, 0, st>>>(w.dBp, w.dBs, ngrp, w.nslices, (int64_t)kQ * N);
-            if ((rc = check_launch("ssd slice_sum_kernel"))) return rc;
-            gs = w.dGs; cs = w.dCs; bs = w.dBs;
+        if (w.ns_g > 1) {
+            slice_sum_kernel<<<(unsigned)ceil_div(ngrp * kQ * kQ / 4, (int64_t)256), 256, 0, st>>>(w.dGp, w.dGs, ngrp, w.ns_g, (int64_t)kQ * kQ);
+            gs = w.dGs;
         }
+        if (w.ns_c > 1) {
+            slice_sum_kernel<<<(unsigned)ceil_div(ngrp * kQ * N / 4, (int64_t)256), 256, 0, st>>>(w.dCp, w.dCs, ngrp, w.ns_c, (int64_t)kQ * N);
+            cs = w.dCs;
+        }
+        if (w.ns_b > 1) {
+            slice_sum_kernel<<<(unsigned)ceil_div(ngrp * kQ * N / 4, (int64_t)256), 256, 0, st>>>(w.dBp, w.dBs, ngrp, w.ns_b, (int64_t)kQ * N);
+            bs = w.dBs;
+        }
+        if ((rc = check_launch("ssd slice_sum_kernel"))) return rc;
         k<<<dim3((unsigned)nc, (unsigned)p->ngroups, (unsigned)p->batch), 512, sm, st>>>(
             gs, cs, bs, static_cast<const T*>(w.Bt), static_cast<const T*>(w.Ct),
             static_cast<T*>(p->dB), static_cast<T*>(p->dC), p->seqlen, p->ngroups, nc,

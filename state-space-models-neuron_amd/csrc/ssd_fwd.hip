@@ -129,7 +129,7 @@ int ssd_fwd_impl(const m2_ssd_params* p, hipStream_t st) {
     a.Z = p->x; a.Z_sb = p->x_stride_b; a.Z_sl = p->x_stride_l; a.Z_sh = p->x_stride_h;
     a.dt_sb = p->dt_stride_b; a.dt_sl = p->dt_stride_l;
     a.seqlen = p->seqlen; a.nheads = p->nheads; a.ngroups = p->ngroups; a.nchunks = nc;
-    ssd_head_slicing(p, 1024, &a.nslices, &a.hps);
+    ssd_slicing(p, kWgsY, &a.nslices, &a.hps);
     a.Y = p->y; a.Y_sb = p->y_stride_b; a.Y_sl = p->y_stride_l; a.Y_sh = p->y_stride_h;
     M2_REQUIRE(p->ngroups * a.nslices <= 65535, M2_ERR_SHAPE, "ssd_fwd: too many group slices");
     const dim3 grid((unsigned)nc, (unsigned)(p->ngroups * a.nslices), (unsigned)p->batch);

@@ -19,33 +19,29 @@ struct SsdWorkspace {
     float* dAp = nullptr; float* dDp = nullptr; float* dBp = nullptr; float* dCp = nullptr; float* dl = nullptr; float* dlc = nullptr; float* dGp = nullptr;
     float* dGs = nullptr; float* dBs = nullptr; float* dCs = nullptr;   // partials summed over the head slices
     float* dirp = nullptr; float* rbp = nullptr; float* dDp8 = nullptr; // per channel-half / per-wave partials of the dx kernel
-    int64_t nslices = 1, heads_per_slice = 1;
+    int64_t ns_g = 1, hps_g = 1, ns_c = 1, hps_c = 1, ns_b = 1, hps_b = 1;   // head slicing of the dg / off<C> / off<B> kernels
     size_t bytes = 0;
 };
 
-// Heads of one group are processed by a workgroup in slices of `heads_per_slice`, so that the
-// group-level dB/dC reductions happen in registers; slices are chosen to give the GPU
-// at least 512 workgroups (two per CU) when the shape allows.
-inline void ssd_bwd_slicing(const m2_ssd_params* p, int64_t* nslices, int64_t* hps) {
-    const int64_t nc = ceil_div(p->seqlen, (int64_t)kQ);
-    const int64_t hpg = p->nheads / p->ngroups;
-    const int64_t base = p->batch * nc * p->ngroups;
-    int64_t best = 1;
-    for (int64_t s = 1; s <= hpg; ++s) {
-        if (hpg % s) continue;
-        best = s;
-        if (base * s >= 512) break;
-    }
-    *nslices = best;
-    *hps = hpg / best;
+// Number of compute units of the current device (queried once per process; 256 on MI355X).
+inline int64_t device_cus() {
+    static int64_t cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        return (int64_t)n;
+    }();
+    return cus;
 }
 
-// Forward / dx kernels: a workgroup loops over `hps` heads of one group (operand fragments shared by the group stay
-// in registers); choose the slice count so that the grid has at least ~1024 workgroups when the shape allows.
-inline void ssd_head_slicing(const m2_ssd_params* p, int64_t target, int64_t* nslices, int64_t* hps) {
+// A workgroup owns one chunk of one group and loops over a slice of that group's heads (operands shared by the
+// group stay on chip, group-level reductions happen in registers).  The slice count is the smallest divisor of
+// heads-per-group that gives at least `wgs_per_cu` workgroups per compute unit: the grid then fills the GPU in one
+// round of long-running workgroups (measured: fewer, longer workgroups beat more, shorter ones for every kernel).
+inline void ssd_slicing(const m2_ssd_params* p, int wgs_per_cu, int64_t* nslices, int64_t* hps) {
     const int64_t nc = ceil_div(p->seqlen, (int64_t)kQ);
     const int64_t hpg = p->nheads / p->ngroups;
     const int64_t base = p->batch * nc * p->ngroups;
+    const int64_t target = device_cus() * wgs_per_cu;
     int64_t best = 1;
     for (int64_t s = 1; s <= hpg; ++s) {
         if (hpg % s) continue;
@@ -55,6 +51,7 @@ inline void ssd_head_slicing(const m2_ssd_params* p, int64_t target, int64_t* ns
     *nslices = best;
     *hps = hpg / best;
 }
+constexpr int kWgsChunkState = 2, kWgsY = 2, kWgsDx = 1, kWgsDg = 1, kWgsOffC = 1, kWgsOffB = 2;
 
 inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd) {
     const int64_t nc = ceil_div(p->seqlen, (int64_t)kQ);
@@ -77,7 +74,9 @@ inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd) {
     w.Bt = take(grp * p->dstate * kQ * esz);
     w.Ct = take(grp * p->dstate * kQ * esz);
     if (bwd) {
-        ssd_bwd_slicing(p, &w.nslices, &w.heads_per_slice);
+        ssd_slicing(p, kWgsDg, &w.ns_g, &w.hps_g);
+        ssd_slicing(p, kWgsOffC, &w.ns_c, &w.hps_c);
+        ssd_slicing(p, kWgsOffB, &w.ns_b, &w.hps_b);
         w.dprev = take(tiles * esz);
         w.dlam = reinterpret_cast<float*>(take(bhc * 4 * kScanSplit));
         w.dAp = reinterpret_cast<float*>(take(bhc * 4));
@@ -87,10 +86,10 @@ inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd) {
         w.dirp = reinterpret_cast<float*>(take(bhc * 2 * kQ * 4));
         w.rbp = reinterpret_cast<float*>(take(bhc * 2 * kQ * 4));
         w.dDp8 = reinterpret_cast<float*>(take(bhc * 8 * 4));
-        w.dGp = reinterpret_cast<float*>(take((size_t)p->batch * nc * p->ngroups * w.nslices * kQ * kQ * 4));
-        const size_t part = (size_t)p->batch * nc * p->ngroups * w.nslices * kQ * p->dstate * 4;
-        w.dBp = reinterpret_cast<float*>(take(part));
-        w.dCp = reinterpret_cast<float*>(take(part));
+        w.dGp = reinterpret_cast<float*>(take((size_t)p->batch * nc * p->ngroups * w.ns_g * kQ * kQ * 4));
+        const size_t part = (size_t)p->batch * nc * p->ngroups * kQ * p->dstate * 4;
+        w.dBp = reinterpret_cast<float*>(take(part * w.ns_b));
+        w.dCp = reinterpret_cast<float*>(take(part * w.ns_c));
         w.dGs = reinterpret_cast<float*>(take((size_t)p->batch * nc * p->ngroups * kQ * kQ * 4));
         w.dBs = reinterpret_cast<float*>(take((size_t)p->batch * nc * p->ngroups * kQ * p->dstate * 4));
         w.dCs = reinterpret_cast<float*>(take((size_t)p->batch * nc * p->ngroups * kQ * p->dstate * 4));
@@ -166,7 +165,7 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
         const size_t sm = state_smem<T, P, N>();
         if ((rc = allow_smem(k, sm))) return rc;
         int64_t ns, hps;
-        ssd_head_slicing(p, 1024, &ns, &hps);
+        ssd_slicing(p, kWgsChunkState, &ns, &hps);
         M2_REQUIRE(p->ngroups * ns <= 65535, M2_ERR_SHAPE, "ssd: too many group slices");
         k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * ns), (unsigned)p->batch), 256, sm, st>>>(
             x, w.ldtab, static_cast<const T*>(w.Bt), w.local, p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
