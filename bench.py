@@ -61,8 +61,8 @@ def bench_ssd(steps, warmup):
     from oracle.ssd import make_ssd_inputs
     cfg = SSD_CFG
     d = make_ssd_inputs(cfg["b"], cfg["l"], cfg["h"], cfg["p"], cfg["n"], cfg["g"], seed=0, dtype=torch.bfloat16, device="cuda:0")
-    # what Mamba2Kernel.forward/backward do: the forward keeps the chunk states for the backward (84 MB here)
-    states = alloc_chunk_states(d["X"], d["B"]) if SAVE_CHUNK_STATES else None
+    # what Mamba2Kernel.forward/backward do: the forward keeps the chunk states and operand tiles for the backward (102 MB here)
+    states = alloc_chunk_states(d["dt"], d["A"], d["X"], d["B"], d["C"]) if SAVE_CHUNK_STATES else None
 
     def step():
         y, _ = ssd_forward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], chunk_states=states)

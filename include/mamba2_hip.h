@@ -91,12 +91,13 @@ int m2_conv1d_bwd(const m2_conv1d_params* p, void* stream);
  * dx, ddt, dB, dC in the dtype of the matching input and dA (h), dD (h) in fp32,
  * already summed over the batch (the reference sums them in its wrapper,
  * mamba2_kernel.py:514).
- * chunk_states (optional): (b, ceil(l/128), h, p, n) elements of `dtype`,
- * m2_ssd_chunk_states_bytes() bytes, 16-byte aligned -- the SSM state entering each chunk.
- * Forward: if non-NULL it is written there (otherwise into the workspace).  Backward: if
- * non-NULL it must hold what the forward wrote for the same inputs and is read instead of
- * being recomputed; with NULL the backward recomputes it from the inputs, as the reference
- * does (mamba2_kernel.py:363-367).
+ * chunk_states (optional): an opaque buffer of m2_ssd_chunk_states_bytes() bytes, 16-byte aligned,
+ * that carries what the backward can reuse from the forward: first the SSM state entering each
+ * chunk, (b, ceil(l/128), h, p, n) elements of `dtype`, then the per-chunk decay tables and the
+ * per-(chunk, group) C B^T operand tiles.  Forward: if non-NULL it is written there (otherwise
+ * into the workspace).  Backward: if non-NULL it must hold what the forward wrote for the same
+ * inputs and is read instead of being recomputed; with NULL the backward recomputes all of it
+ * from the inputs, as the reference does (mamba2_kernel.py:363-367).
  */
 typedef struct m2_ssd_params {
     const void* x; const void* dt; const float* A; const void* B; const void* C; const float* D;

@@ -306,16 +306,23 @@ off_kernel(const T* __restrict__ Arow, int64_t Asb, int64_t Asl, int64_t Ash,   
             out[(rb * 32 + acc_row(lane, v)) * N + (nb0 + jn) * 32 + r] = acc[0][jn][v];
 }
 
-// Sum of the per-slice partials (fixed order).  One thread per float4; `tile` floats per (group, slice) tile.
+// Sum of the per-slice partials (fixed order) of up to three arrays in one launch.  One thread per float4;
+// `tile` floats per (group, slice) tile; segment k covers threads [first_k, first_{k+1}).
+struct SliceSumSeg { const float* part; float* out; int64_t nslices, tile, first; };
+struct SliceSumArgs { SliceSumSeg seg[3]; int nseg; int64_t total; };
 __global__ void __launch_bounds__(256)
-slice_sum_kernel(const float* __restrict__ part, float* __restrict__ out, int64_t ngrp, int64_t nslices, int64_t tile) {
+slice_sum_kernel(const SliceSumArgs a) {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t per = tile / 4;
-    if (idx >= ngrp * per) return;
-    const int64_t grp = idx / per, e = (idx % per) * 4;
+    if (idx >= a.total) return;
+    int k = 0;
+    if (a.nseg > 1 && idx >= a.seg[1].first) k = 1;
+    if (a.nseg > 2 && idx >= a.seg[2].first) k = 2;
+    const SliceSumSeg sg = a.seg[k];
+    const int64_t per = sg.tile / 4, loc = idx - sg.first;
+    const int64_t grp = loc / per, e = (loc % per) * 4;
     floatx4 s = {0.f, 0.f, 0.f, 0.f};
-    for (int64_t sl = 0; sl < nslices; ++sl) s += *reinterpret_cast<const floatx4*>(part + (grp * nslices + sl) * tile + e);
-    *reinterpret_cast<floatx4*>(out + grp * tile + e) = s;
+    for (int64_t sl = 0; sl < sg.nslices; ++sl) s += *reinterpret_cast<const floatx4*>(sg.part + (grp * sg.nslices + sl) * sg.tile + e);
+    *reinterpret_cast<floatx4*>(sg.out + grp * sg.tile + e) = s;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -461,8 +468,8 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
     const dim3 grid_b((unsigned)nc, (unsigned)(p->ngroups * w.ns_b), (unsigned)p->batch);
     M2_REQUIRE(p->nheads <= 65535, M2_ERR_SHAPE, "ssd_bwd: too many group slices");
     int rc;
-    // G (+ operand tiles); the state entering each chunk, unless the caller kept the forward's
-    if ((rc = ssd_launch_states<T, P, N>(p, w, nullptr, st, p->chunk_states != nullptr))) return rc;
+    // decay tables, G (+ operand tiles) and the state entering each chunk, unless the caller kept the forward's
+    if (!p->chunk_states && (rc = ssd_launch_states<T, P, N>(p, w, nullptr, st))) return rc;
     // local dS contributions (reuses the `local` region) and the reverse recurrence
     {
         auto k = chunk_state_kernel<T, P, N, true>;
@@ -536,9 +543,9 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
             const Dx16Out o{w.dirp, w.rbp, w.dDp8};
             k<<<grid, 512, sm, st>>>(a, o);
             if ((rc = check_launch("ssd_dx16_kernel"))) return rc;
-            da_kernel<T><<<(unsigned)(p->batch * p->nheads * nc), 64, 0, st>>>(
+            da_kernel<T><<<(unsigned)ceil_div(p->batch * p->nheads * nc, (int64_t)4), 256, 0, st>>>(
                 p->dt, dt_f32, p->dt_stride_b, p->dt_stride_l, p->A, w.dl, w.dlc, w.dlam, w.dirp, w.rbp, w.dDp8,
-                p->ddt, p->ddt_stride_b, p->ddt_stride_l, w.dAp, w.dDp, p->seqlen, p->nheads, nc);
+                p->ddt, p->ddt_stride_b, p->ddt_stride_l, w.dAp, w.dDp, p->seqlen, p->nheads, nc, p->batch * p->nheads * nc);
             if ((rc = check_launch("ssd da_kernel"))) return rc;
         } else {
             auto k = diag_off_kernel<T, P, N, true>;
@@ -554,17 +561,20 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         if ((rc = allow_smem(k, sm))) return rc;
         const int64_t ngrp = p->batch * nc * p->ngroups;
         const float *gs = w.dGp, *cs = w.dCp, *bs = w.dBp;
-        if (w.ns_g > 1) {
-            slice_sum_kernel<<<(unsigned)ceil_div(ngrp * kQ * kQ / 4, (int64_t)256), 256, 0, st>>>(w.dGp, w.dGs, ngrp, w.ns_g, (int64_t)kQ * kQ);
-            gs = w.dGs;
-        }
-        if (w.ns_c > 1) {
-            slice_sum_kernel<<<(unsigned)ceil_div(ngrp * kQ * N / 4, (int64_t)256), 256, 0, st>>>(w.dCp, w.dCs, ngrp, w.ns_c, (int64_t)kQ * N);
-            cs = w.dCs;
-        }
-        if (w.ns_b > 1) {
-            slice_sum_kernel<<<(unsigned)ceil_div(ngrp * kQ * N / 4, (int64_t)256), 256, 0, st>>>(w.dBp, w.dBs, ngrp, w.ns_b, (int64_t)kQ * N);
-            bs = w.dBs;
+        {
+            SliceSumArgs sa{};
+            int64_t first = 0;
+            auto add = [&](const float* part, float* out, int64_t ns, int64_t tile, const float** use) {
+                if (ns <= 1) return;
+                sa.seg[sa.nseg++] = SliceSumSeg{part, out, ns, tile, first};
+                first += ngrp * tile / 4;
+                *use = out;
+            };
+            add(w.dGp, w.dGs, w.ns_g, (int64_t)kQ * kQ, &gs);
+            add(w.dCp, w.dCs, w.ns_c, (int64_t)kQ * N, &cs);
+            add(w.dBp, w.dBs, w.ns_b, (int64_t)kQ * N, &bs);
+            sa.total = first;
+            if (sa.nseg > 0) slice_sum_kernel<<<(unsigned)ceil_div(first, (int64_t)256), 256, 0, st>>>(sa);
         }
         if ((rc = check_launch("ssd slice_sum_kernel"))) return rc;
         k<<<dim3((unsigned)nc, (unsigned)p->ngroups, (unsigned)p->batch), 512, sm, st>>>(

@@ -274,18 +274,19 @@ ssd_dx16_kernel(const DiagArgs a, const Dx16Out o) {
 }
 
 // Per (batch, head, chunk): da_t = sum_{i>=t} (dl_diag_i + dl_c_i) + sum_{j<t} rb_j + dlam,  ddt_t = A da_t + dir_t,
-// dA partial = sum_t da_t dt_t, dD partial = sum of the eight per-wave partials.  One wave per (b, h, c); lanes hold
+// dA partial = sum_t da_t dt_t, dD partial = sum of the eight per-wave partials.  One wave per (b, h, c), four per workgroup; lanes hold
 // the tokens in reverse order (127 - lane, 63 - lane), so the suffix over tokens is an inclusive prefix over lanes and
 // the exclusive prefix over tokens an exclusive suffix over lanes.
 template <typename T>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(256)
 da_kernel(const void* __restrict__ dt, int dt_f32, int64_t dt_sb, int64_t dt_sl, const float* __restrict__ A,
           const float* __restrict__ dl_diag, const float* __restrict__ dl_c, const float* __restrict__ dlam,
           const float* __restrict__ dirp, const float* __restrict__ rbp, const float* __restrict__ dDp8,
           void* __restrict__ ddt, int64_t ddt_sb, int64_t ddt_sl, float* __restrict__ dAp, float* __restrict__ dDp,
-          int64_t seqlen, int64_t nheads, int64_t nchunks) {
-    const int lane = threadIdx.x;
-    const int64_t bhc = blockIdx.x;
+          int64_t seqlen, int64_t nheads, int64_t nchunks, int64_t total) {
+    const int lane = threadIdx.x & 63;
+    const int64_t bhc = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (bhc >= total) return;
     const int64_t c = bhc % nchunks, h = (bhc / nchunks) % nheads, b = bhc / (nchunks * nheads);
     const int64_t t0 = c * kQ;
     const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);

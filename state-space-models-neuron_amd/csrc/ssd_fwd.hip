@@ -152,8 +152,7 @@ int ssd_fwd_impl(const m2_ssd_params* p, hipStream_t st) {
 
 extern "C" size_t m2_ssd_chunk_states_bytes(const m2_ssd_params* p) {
     if (!p || p->batch <= 0 || p->seqlen <= 0 || p->nheads <= 0) return 0;
-    const int64_t nc = m2::ceil_div(p->seqlen, (int64_t)m2::kQ);
-    return (size_t)p->batch * nc * p->nheads * p->headdim * p->dstate * (p->dtype == M2_F32 ? 4 : 2);
+    return m2::ssd_carve(p, nullptr, false, true).kept_bytes;
 }
 
 extern "C" size_t m2_ssd_fwd_workspace_bytes(const m2_ssd_params* p) {

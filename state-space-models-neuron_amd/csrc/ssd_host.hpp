@@ -21,6 +21,7 @@ struct SsdWorkspace {
     float* dirp = nullptr; float* rbp = nullptr; float* dDp8 = nullptr; // per channel-half / per-wave partials of the dx kernel
     int64_t ns_g = 1, hps_g = 1, ns_c = 1, hps_c = 1, ns_b = 1, hps_b = 1;   // head slicing of the dg / off<C> / off<B> kernels
     size_t bytes = 0;
+    size_t kept_bytes = 0;              // size of the forward -> backward carry-over (chunk_states buffer)
 };
 
 // Number of compute units of the current device (queried once per process; 256 on MI355X).
@@ -53,7 +54,7 @@ inline void ssd_slicing(const m2_ssd_params* p, int wgs_per_cu, int64_t* nslices
 }
 constexpr int kWgsChunkState = 2, kWgsY = 2, kWgsDx = 1, kWgsDg = 1, kWgsOffC = 1, kWgsOffB = 2;
 
-inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd) {
+inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd, bool kept_only = false) {
     const int64_t nc = ceil_div(p->seqlen, (int64_t)kQ);
     const size_t esz = p->dtype == M2_F32 ? 4 : 2;
     const size_t tiles = (size_t)p->batch * nc * p->nheads * p->headdim * p->dstate;
@@ -62,17 +63,30 @@ inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd) {
     SsdWorkspace w;
     unsigned char* b8 = static_cast<unsigned char*>(base);
     auto take = [&](size_t n) { unsigned char* r = b8 ? b8 + off : nullptr; off += align_up(n, 256); return r; };
-    w.G = reinterpret_cast<float*>(take((size_t)p->batch * nc * p->ngroups * kQ * kQ * 4));
     w.local = reinterpret_cast<float*>(take(tiles * 4));
-    if (p->chunk_states) w.prev = p->chunk_states;      // caller keeps the chunk states (forward -> backward)
-    else w.prev = take(tiles * esz);
-    w.lam = reinterpret_cast<float*>(take(bhc * 4));
-    w.ldtab = reinterpret_cast<float*>(take(bhc * 2 * kQ * 4));
-    const size_t grp = (size_t)p->batch * nc * p->ngroups;
-    w.Gm = take(grp * kQ * kQ * esz);
-    w.Gmt = take(grp * kQ * kQ * esz);
-    w.Bt = take(grp * p->dstate * kQ * esz);
-    w.Ct = take(grp * p->dstate * kQ * esz);
+    // What the backward reuses from the forward: the state entering each chunk, the decay tables and the
+    // per-(chunk, group) operand tiles.  They live in the caller's chunk_states buffer when one is given
+    // (forward writes, backward reads), otherwise in the workspace (backward recomputes them).
+    {
+        size_t koff = 0;
+        unsigned char* k8 = static_cast<unsigned char*>(p->chunk_states);
+        auto keep = [&](size_t n) -> unsigned char* {
+            if (!p->chunk_states && !kept_only) return take(n);
+            unsigned char* r = k8 ? k8 + koff : nullptr;
+            koff += align_up(n, 256);
+            return r;
+        };
+        const size_t grp = (size_t)p->batch * nc * p->ngroups;
+        w.prev = keep(tiles * esz);
+        w.lam = reinterpret_cast<float*>(keep(bhc * 4));
+        w.ldtab = reinterpret_cast<float*>(keep(bhc * 2 * kQ * 4));
+        w.G = reinterpret_cast<float*>(keep(grp * kQ * kQ * 4));
+        w.Gm = keep(grp * kQ * kQ * esz);
+        w.Gmt = keep(grp * kQ * kQ * esz);
+        w.Bt = keep(grp * p->dstate * kQ * esz);
+        w.Ct = keep(grp * p->dstate * kQ * esz);
+        w.kept_bytes = koff;
+    }
     if (bwd) {
         ssd_slicing(p, kWgsDg, &w.ns_g, &w.hps_g);
         ssd_slicing(p, kWgsOffC, &w.ns_c, &w.hps_c);
@@ -134,10 +148,10 @@ inline size_t state_smem() { return (size_t)(P + N) * lds_ld<T>(kQ) * sizeof(T);
 template <typename T>
 inline size_t cb_smem() { return (size_t)2 * kQ * lds_ld<T>(64) * sizeof(T); }
 
-// G = C B^T, local chunk states, forward state scan.  Used by the forward and (recompute) by the backward;
-// `cb_only` stops after the first (the backward was handed the chunk states).
+// Decay tables, G = C B^T (+ operand tiles), local chunk states, forward state scan.  Used by the forward and, when the
+// caller did not keep the forward's chunk_states buffer, by the backward (recompute).
 template <typename T, int P, int N>
-inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, float* final_out, hipStream_t st, bool cb_only = false) {
+inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, float* final_out, hipStream_t st) {
     const int64_t nc = ceil_div(p->seqlen, (int64_t)kQ);
     const T* x = static_cast<const T*>(p->x);
     const T* Bm = static_cast<const T*>(p->B);
@@ -159,7 +173,6 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
             p->C_stride_b, p->C_stride_l, p->C_stride_g);
         if ((rc = check_launch("ssd cb_kernel"))) return rc;
     }
-    if (cb_only) return M2_OK;
     {
         auto k = chunk_state_kernel<T, P, N, false>;
         const size_t sm = state_smem<T, P, N>();

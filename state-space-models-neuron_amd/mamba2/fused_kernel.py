@@ -51,7 +51,7 @@ def _forward_parts(zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, n_groups, d
     dt_sp = glue.softplus_bias(dt, dt_bias)
     x, Bm, Cm = _xbc_views(conv_out, n_groups, d_state, d_inner, d_head)
     # the scan's chunk states are kept for the backward when one follows directly (no second recompute there)
-    states = alloc_chunk_states(x, Bm) if (keep_states and x.numel() > 0) else None
+    states = alloc_chunk_states(dt_sp, logA, x, Bm, Cm) if (keep_states and x.numel() > 0) else None
     y, _ = ssd_forward(dt_sp, logA, x, Bm, Cm, D, chunk_states=states)
     scan_out = y.view(b, l, d_inner)
     norm_out = glue.rmsnorm_gated(scan_out, z, norm_w, n_groups, NORM_EPS, out_dtype=zxBCdt.dtype)

@@ -60,11 +60,14 @@ def _validate(dt, A, X, B, C, D, initial_state):
     _lib.require_gpu(dt, A, X, B, C, D, initial_state)
 
 
-def alloc_chunk_states(X, B):
-    """Buffer for the SSM state entering each 128-token chunk, (b, ceil(l/128), h, p, n) in X's dtype:
-    filled by ``ssd_forward(..., chunk_states=buf)`` and consumed by ``ssd_backward(..., chunk_states=buf)``."""
-    b, l, h, hd = X.shape
-    return torch.empty((b, -(-l // 128), h, hd, B.shape[3]), dtype=X.dtype, device=X.device)
+def alloc_chunk_states(dt, A, X, B, C):
+    """Carry-over buffer from ``ssd_forward(..., chunk_states=buf)`` to ``ssd_backward(..., chunk_states=buf)``
+    (opaque bytes): the SSM state entering each 128-token chunk -- the first b*ceil(l/128)*h*p*n elements, in
+    X's dtype -- followed by the decay tables and the per-chunk operand tiles."""
+    lib = _lib.load()
+    p = SsdParams()
+    _fill_common(p, dt, A, X, B, C, None)
+    return torch.empty(lib.m2_ssd_chunk_states_bytes(p), dtype=torch.uint8, device=X.device)
 
 
 def ssd_forward(dt, A, X, B, C, D=None, initial_state=None, want_final_state=False, chunk_states=None):
@@ -95,9 +98,8 @@ def _chunk_states_ptr(lib, p, chunk_states):
     if chunk_states is None:
         return None
     need = lib.m2_ssd_chunk_states_bytes(p)
-    if not chunk_states.is_contiguous() or chunk_states.numel() * chunk_states.element_size() != need or \
-            _lib.dtype_code(chunk_states.dtype) != p.dtype:
-        raise ValueError(f"chunk_states must be a contiguous buffer of {need} bytes in the dtype of X (see alloc_chunk_states)")
+    if not chunk_states.is_contiguous() or chunk_states.numel() * chunk_states.element_size() != need:
+        raise ValueError(f"chunk_states must be a contiguous buffer of {need} bytes (see alloc_chunk_states)")
     return ptr(chunk_states)
 
 
@@ -160,7 +162,7 @@ class Mamba2Kernel(torch.autograd.Function):
     @staticmethod
     def forward(ctx, dt, A, X, B, C, D, initial_state=None, return_final_state=False):
         needs_grad = any(ctx.needs_input_grad[:7])
-        states = alloc_chunk_states(X, B) if (SAVE_CHUNK_STATES and needs_grad and X.numel() > 0) else None
+        states = alloc_chunk_states(dt, A, X, B, C) if (SAVE_CHUNK_STATES and needs_grad and X.numel() > 0) else None
         Y, S = ssd_forward(dt, A, X, B, C, D, initial_state, return_final_state, chunk_states=states)
         ctx.chunk_states = states
         ctx.save_for_backward(dt, A, X, B, C, D, initial_state)

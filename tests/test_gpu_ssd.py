@@ -164,15 +164,16 @@ def test_ssd_backward_kept_chunk_states_equal_recompute(dtype):
     b, l, h, p, n, g = 2, 300, 4, 64, 128, 2
     d = _dev(make_ssd_inputs(b, l, h, p, n, g, seed=21, dtype=dtype))
     S0 = 0.1 * torch.randn(b, h, p, n, generator=torch.Generator().manual_seed(5)).to(DEV)
-    states = alloc_chunk_states(d["X"], d["B"])
-    assert states.shape == (b, 3, h, p, n) and states.dtype == dtype
+    states = alloc_chunk_states(d["dt"], d["A"], d["X"], d["B"], d["C"])
+    assert states.dtype == torch.uint8 and states.numel() >= b * 3 * h * p * n * d["X"].element_size()
     y1, _ = ssd_forward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], S0, chunk_states=states)
     y0, _ = ssd_forward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], S0)
     assert torch.equal(y0, y1)
-    assert torch.equal(states[:, 0].float(), S0.to(dtype).float())      # the state entering chunk 0 is the initial state
+    first = states[:b * 3 * h * p * n * d["X"].element_size()].view(dtype).view(b, 3, h, p, n)
+    assert torch.equal(first[:, 0].float(), S0.to(dtype).float())      # the state entering chunk 0 is the initial state
     g0 = ssd_backward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], d["dy"], S0, want_dinitial=True)
     g1 = ssd_backward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], d["dy"], S0, want_dinitial=True, chunk_states=states)
     for a_, b_ in zip(g0, g1):
         assert torch.equal(a_, b_)
     with pytest.raises(ValueError, match="chunk_states"):
-        ssd_backward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], d["dy"], chunk_states=states[:, :2].contiguous())
+        ssd_backward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], d["dy"], chunk_states=states[:-256].contiguous())
