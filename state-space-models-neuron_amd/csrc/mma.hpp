@@ -79,6 +79,17 @@ __device__ __forceinline__ Frag<float> scale_frag(const Frag<float>& a, const fl
     return r;
 }
 
+// Makes a fragment opaque to the optimiser at this point (no instruction is emitted).  Used on loop-invariant
+// fragments that are re-scaled inside a loop: without it the bf16 -> fp32 unpacking of the fragment is hoisted out of
+// the loop and the fragment then occupies eight fp32 registers instead of four packed ones for the whole loop.
+__device__ __forceinline__ void keep_packed(Frag<bf16_t>& f) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 raw = __builtin_bit_cast(u32x4, f.v);
+    asm volatile("" : "+v"(raw));
+    f.v = __builtin_bit_cast(bf16x8, raw);
+}
+__device__ __forceinline__ void keep_packed(Frag<float>&) {}
+
 // One wave: acc[i][j] (32x32 blocks) += A[rows i*32.., k0:k1] * Bt[rows j*32.., k0:k1]^T, operands in LDS.
 // A points at the first of this wave's BM*32 rows, Bt at the first of its BN*32 rows.  k0, k1 multiples of 16.
 template <int BM, int BN, typename T>

@@ -507,6 +507,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         if ((rc = check_launch("ssd dg_kernel"))) return rc;
     }
     {
+        if constexpr (!bwd16_ok<T, P, N>()) {
         auto kc = off_kernel<T, P, N, true>;
         auto kb = off_kernel<T, P, N, false>;
         const size_t smc = off_smem<T, P, N>(true), sm = off_smem<T, P, N>(false);
@@ -520,6 +521,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
                                     static_cast<const T*>(w.dprev), nullptr, 0, 0, 0,
                                     w.dBp, nullptr, p->seqlen, p->nheads, p->ngroups, nc, w.ns_b, w.hps_b);
         if ((rc = check_launch("ssd off_kernel<B>"))) return rc;
+        }
     }
     {
         DiagArgs a{};
@@ -529,23 +531,33 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         a.Z = p->dy; a.Z_sb = p->dy_stride_b; a.Z_sl = p->dy_stride_l; a.Z_sh = p->dy_stride_h;
         a.dt_sb = p->dt_stride_b; a.dt_sl = p->dt_stride_l;
         a.seqlen = p->seqlen; a.nheads = p->nheads; a.ngroups = p->ngroups; a.nchunks = nc;
-        ssd_slicing(p, dx16_ok<T, P, N>() ? kWgsDx : 2, &a.nslices, &a.hps);
+        ssd_slicing(p, 2, &a.nslices, &a.hps);
         a.X = p->x; a.X_sb = p->x_stride_b; a.X_sl = p->x_stride_l; a.X_sh = p->x_stride_h;
         a.dX = p->dx; a.dX_sb = p->dx_stride_b; a.dX_sl = p->dx_stride_l; a.dX_sh = p->dx_stride_h;
         a.ddt = p->ddt; a.ddt_sb = p->ddt_stride_b; a.ddt_sl = p->ddt_stride_l;
         a.ldtab = w.ldtab;
         a.dl_diag = w.dl; a.dl_c = w.dlc; a.dlam = w.dlam; a.dAp = w.dAp; a.dDp = w.dDp;
         const dim3 grid((unsigned)nc, (unsigned)(p->ngroups * a.nslices), (unsigned)p->batch);
-        if constexpr (dx16_ok<T, P, N>()) {
-            auto k = ssd_dx16_kernel<T, P, N>;
-            const size_t sm = dx16_smem<P, N>();
+        if constexpr (bwd16_ok<T, P, N>()) {
+            Bwd16Args m{};
+            m.ldtab = w.ldtab; m.D = p->D;
+            m.Bm = p->B; m.B_sb = p->B_stride_b; m.B_sl = p->B_stride_l; m.B_sg = p->B_stride_g;
+            m.Cm = p->C; m.C_sb = p->C_stride_b; m.C_sl = p->C_stride_l; m.C_sg = p->C_stride_g;
+            m.Gmt = w.Gmt; m.dS = w.dprev; m.Sprev = w.prev;
+            m.dy = p->dy; m.dy_sb = p->dy_stride_b; m.dy_sl = p->dy_stride_l; m.dy_sh = p->dy_stride_h;
+            m.x = p->x; m.x_sb = p->x_stride_b; m.x_sl = p->x_stride_l; m.x_sh = p->x_stride_h;
+            m.dx = p->dx; m.dx_sb = p->dx_stride_b; m.dx_sl = p->dx_stride_l; m.dx_sh = p->dx_stride_h;
+            m.dirp = w.dirp; m.rbp = w.rbp; m.dlc = w.dlc; m.dDp8 = w.dDp8; m.dBp = w.dBp; m.dCp = w.dCp;
+            m.seqlen = p->seqlen; m.nheads = p->nheads; m.ngroups = p->ngroups; m.nchunks = nc;
+            m.nslices = w.ns_b; m.hps = w.hps_b;
+            auto k = ssd_bwd16_kernel<T, P, N>;
+            const size_t sm = bwd16_smem<P, N>();
             if ((rc = allow_smem(k, sm))) return rc;
-            const Dx16Out o{w.dirp, w.rbp, w.dDp8};
-            k<<<grid, 512, sm, st>>>(a, o);
-            if ((rc = check_launch("ssd_dx16_kernel"))) return rc;
+            k<<<grid_b, 512, sm, st>>>(m);
+            if ((rc = check_launch("ssd_bwd16_kernel"))) return rc;
             da_kernel<T><<<(unsigned)ceil_div(p->batch * p->nheads * nc, (int64_t)4), 256, 0, st>>>(
-                p->dt, dt_f32, p->dt_stride_b, p->dt_stride_l, p->A, w.dl, w.dlc, w.dlam, w.dirp, w.rbp, w.dDp8,
-                p->ddt, p->ddt_stride_b, p->ddt_stride_l, w.dAp, w.dDp, p->seqlen, p->nheads, nc, p->batch * p->nheads * nc);
+                w.ldtab, p->A, w.dl, w.dlc, w.dlam, w.dirp, w.rbp, w.dDp8,
+                p->ddt, dt_f32, p->ddt_stride_b, p->ddt_stride_l, w.dAp, w.dDp, p->seqlen, p->nheads, nc, p->batch * p->nheads * nc);
             if ((rc = check_launch("ssd da_kernel"))) return rc;
         } else {
             auto k = diag_off_kernel<T, P, N, true>;

@@ -1,0 +1,465 @@
+// SSD backward main kernel for 16-bit operands: dx, the per-token decay-gradient terms, and the state parts of dB and
+// dC, from ONE pass over dy, x, dS (gradient of the state leaving the chunk) and S_prev (state entering it).
+//
+// A workgroup of 8 waves handles one chunk of one group and loops over `hps` heads.  Per head the four tiles --
+// dS [P][N], S_prev [P][N], dy [128][P], x [128][P] -- and the [ l | dt ] table are copied global -> LDS
+// asynchronously, one head ahead, into one of two buffers (one barrier per head); all tiles keep their global layout
+// (slots XOR-swizzled inside each row) and reach the MFMA either row-wise or through LDS transpose reads.
+//
+// The waves are specialised by role, two per 32-token row block (so that each role's long-lived registers are its own):
+//   role A (waves 0-3): dxd[j][p] = u_j ( e^{Lam-l_ref} sum_n B[j][n] dS[p][n] + sum_{i>=j} (G[i][j] v_i) dy[i][p] )
+//            dx = dt_j dxd + D dy,   dir_j = sum_p dxd x,   rb_j = dt_j sum_p (state part of dxd) x,
+//            dl_c[i] = e^{l_i} sum_p dy[i][p] (sum_n C[i][n] S_prev[p][n]),   dD partial = sum dy x
+//            (B rows, C rows and the transposed causal C B^T rows of its tokens stay on chip: registers, and for half of
+//            the C fragments a wave-private LDS tile)
+//   role B (waves 4-7):  dB_off[j][n] += dt_j e^{Lam-l_j} sum_p x[j][p] dS[p][n]
+//                        dC_off[i][n] += e^{l_i}          sum_p dy[i][p] S_prev[p][n]
+//            accumulated over the workgroup's heads in registers (row scale applied in fp32 after the MFMA, so both
+//            operands are exact copies of the inputs) and written once at the end.
+// The decay is factorised per row block around its LAST token (see ssd_diag.hpp), with the exact per-element
+// fallback when the block's range exceeds kMaxRange.  ddt and dA need a scan over the chunk and are left to da_kernel.
+#pragma once
+#include "ssd_y.hpp"
+
+namespace m2 {
+
+// of the N / 16 C-row fragments a role-A wave needs, this many live in a wave-private LDS tile instead of registers
+template <int N> constexpr int bwd16_clds() { return N / 16 > 4 ? N / 32 : 0; }
+template <int P, int N>
+constexpr size_t bwd16_smem() {
+    return (size_t)2 * ((2 * P * N + 2 * kQ * P) * 2 + 2 * kQ * sizeof(float)) + (size_t)4 * (kQ + 32) * sizeof(float) + (size_t)4 * 8 * P * sizeof(float) +
+           (size_t)4 * 32 * (bwd16_clds<N>() * 16 + 8) * 2;
+}
+template <typename T, int P, int N>
+constexpr bool bwd16_ok() { return sizeof(T) == 2 && bwd16_smem<P, N>() <= 160 * 1024; }
+
+struct Bwd16Args {
+    const float* ldtab;                                   // [b][h][c][ l kQ | dt kQ ]
+    const float* D;
+    const void* Bm; int64_t B_sb, B_sl, B_sg;             // B, C: [b][l][g][N]
+    const void* Cm; int64_t C_sb, C_sl, C_sg;
+    const void* Gmt;                                      // (causal C B^T)^T: [b][c][g][kQ][kQ]
+    const void* dS; const void* Sprev;                    // [b][c][h][P][N]
+    const void* dy; int64_t dy_sb, dy_sl, dy_sh;
+    const void* x; int64_t x_sb, x_sl, x_sh;
+    void* dx; int64_t dx_sb, dx_sl, dx_sh;
+    float* dirp; float* rbp; float* dlc;                  // [b][h][c][kQ]
+    float* dDp8;                                          // [b][h][c][8]
+    float* dBp; float* dCp;                               // [b][c][g][slice][kQ][N]
+    int64_t seqlen, nheads, ngroups, nchunks, nslices, hps;
+};
+
+template <typename T, int P, int N>
+__global__ void __launch_bounds__(512, 1)
+ssd_bwd16_kernel(const Bwd16Args a) {
+    static_assert(sizeof(T) == 2, "16-bit operands only");
+    constexpr int BN = P / 32, KSN = N / 16, KSP = P / 16, NBN = N / 32;
+    constexpr int SPR_S = N / 8, SPR_X = P / 8;
+    constexpr int NS = P * SPR_S / 512, NX = kQ * SPR_X / 512;
+    constexpr int TAB = kQ + 32;
+    constexpr int TILES = 2 * P * N + 2 * kQ * P;    // elements per buffer
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* tiles = reinterpret_cast<T*>(smem_raw);                       // [2][ dS | S_prev | dy | x ]
+    float* sLD = reinterpret_cast<float*>(tiles + 2 * TILES);        // [2][ l kQ | dt kQ ]
+    float* wt_all = sLD + 2 * 2 * kQ;                                // [4 role-A waves][wv kQ | wu 32]
+    float* sY = wt_all + 4 * TAB;                                    // [4 role-A waves][8][P]
+    constexpr int KCL = bwd16_clds<N>(), KCR = KSN - KCL;            // C-row fragments in LDS / in registers
+    constexpr int LDC = KCL * 16 + 8;
+    T* sFC = reinterpret_cast<T*>(sY + 4 * 8 * P);                   // [4 role-A waves][32][LDC]
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 31, half = lane >> 5;
+    const int rbk = wave & 3, role = wave >> 2;      // waves w and w + 4 share a SIMD: one of each role per SIMD
+    const int64_t c = blockIdx.x, b = blockIdx.z;
+    const int64_t g = blockIdx.y / a.nslices, slice = blockIdx.y % a.nslices;
+    const int64_t hpg = a.nheads / a.ngroups;
+    const int64_t t0 = c * kQ;
+    const int valid = (int)((a.seqlen - t0) < kQ ? (a.seqlen - t0) : kQ);
+    const int row0 = rbk * 32;
+    const int64_t h_first = g * hpg + slice * a.hps;
+    // transpose-read lane roles: the 16 lanes of a group fetch a [4 rows][16 columns] block; lane (i0 = bits 3:2, i1 = bits 1:0)
+    // supplies the address of row i0, columns 4 i1 .. 4 i1 + 3 and receives column (lane & 15) of rows 0..3
+    const int tr_row = (lane >> 2) & 3;
+    const int tr_col = ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+    typedef T tvec4 __attribute__((ext_vector_type(4)));
+
+    const uint32_t wave_u = uniform(wave), lds_T = uniform(lds_addr_of(tiles)), lds_LD = uniform(lds_addr_of(sLD));
+    auto issue_tiles = [&](int64_t h, int buf) {
+        const int64_t tile = ((b * a.nchunks + c) * a.nheads + h) * (int64_t)(P * N);
+        const T* Sp = static_cast<const T*>(a.dS) + tile;
+        const T* Pp = static_cast<const T*>(a.Sprev) + tile;
+        const uint32_t dst = lds_T + (uint32_t)(buf * TILES * 2);
+        // the per-lane source offsets are recomputed for every head on purpose (a handful of integer instructions):
+        // kept in registers across the head loop they are the first thing the register allocator spills, and a
+        // spill reload in the middle of this sequence waits for all copies issued so far
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+#pragma unroll
+        for (int it = 0; it < NS; ++it) {
+            const int s = (int)(wave_u * NS + it) * 64 + ln;
+            const int row = s / SPR_S, cs = (s % SPR_S) ^ swz_s<SPR_S>(row);
+            const uint32_t off = (uint32_t)(row * N + cs * 8) * 2u;
+            async_copy16(Sp, off, dst + (wave_u * NS + it) * 1024u);
+            async_copy16(Pp, off, dst + (uint32_t)(P * N * 2) + (wave_u * NS + it) * 1024u);
+        }
+        const T* Yp = static_cast<const T*>(a.dy) + b * a.dy_sb + t0 * a.dy_sl + h * a.dy_sh;
+        const T* Xp = static_cast<const T*>(a.x) + b * a.x_sb + t0 * a.x_sl + h * a.x_sh;
+#pragma unroll
+        for (int it = 0; it < NX; ++it) {
+            const int s = (int)(wave_u * NX + it) * 64 + ln;
+            const int row = s / SPR_X, cs = (s % SPR_X) ^ swz_x(row);
+            const int grow = row < valid ? row : valid - 1;       // rows past the end: finite stand-ins, masked by zero scales
+            async_copy16(Yp, (uint32_t)(grow * a.dy_sl + cs * 8) * 2u, dst + (uint32_t)(2 * P * N * 2) + (wave_u * NX + it) * 1024u);
+            async_copy16(Xp, (uint32_t)(grow * a.x_sl + cs * 8) * 2u, dst + (uint32_t)((2 * P * N + kQ * P) * 2) + (wave_u * NX + it) * 1024u);
+        }
+        async_copy_ldtab(a.ldtab, (b * a.nheads + h) * a.nchunks + c, lds_LD + (uint32_t)(buf * 2 * kQ * 4));
+    };
+    issue_tiles(h_first, 0);
+
+    if (role == 0) {
+        // =============================================================== role A: dx, dir, rb, dl_c, dD
+        float* wv = wt_all + rbk * TAB;
+        float* wu = wv + kQ;
+        float* sYw = sY + rbk * 8 * P;
+        T* sFCw = sFC + rbk * 32 * LDC;
+        Frag<T> fd[8], foB[KSN], foC[KCR];
+        {
+            const T* Gp = static_cast<const T*>(a.Gmt) + ((b * a.nchunks + c) * a.ngroups + g) * (int64_t)(kQ * kQ) + (row0 + r) * kQ;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks)
+                if (ks >= 2 * rbk) fd[ks] = load_frag(Gp + ks * 16 + half * 8);
+            const T* Bp = static_cast<const T*>(a.Bm) + b * a.B_sb + (t0 + row0 + r) * a.B_sl + g * a.B_sg;
+            const T* Cp = static_cast<const T*>(a.Cm) + b * a.C_sb + (t0 + row0 + r) * a.C_sl + g * a.C_sg;
+            const bool ok = row0 + r < valid;
+#pragma unroll
+            for (int ks = 0; ks < KSN; ++ks) {
+                Frag<T> fc;
+                if (ok) { foB[ks] = load_frag(Bp + ks * 16 + half * 8); fc = load_frag(Cp + ks * 16 + half * 8); }
+                else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) { foB[ks].v[e] = (T)0.f; fc.v[e] = (T)0.f; }
+                }
+                if (ks < KCR) foC[ks < KCR ? ks : 0] = fc;
+                else *reinterpret_cast<bf16x8*>(sFCw + r * LDC + (ks - KCR) * 16 + half * 8) = fc.v;     // read back by the same lane only
+            }
+        }
+        for (int64_t hh = 0; hh < a.hps; ++hh) {
+            const int64_t h = h_first + hh;
+            const int buf = (int)(hh & 1);
+            const int64_t bhc = (b * a.nheads + h) * a.nchunks + c;
+            const float Dh = a.D ? a.D[h] : 0.f;
+
+            wait_vmem_all();          // this wave's share of the tiles of head hh, and the whole [ l | dt ] table, have landed
+            const float* sl = sLD + buf * 2 * kQ;
+            const float* sd = sl + kQ;
+            const float l_first = sl[row0], l_last = sl[row0 + 31], Lam = sl[kQ - 1];
+            const bool fast = (l_first - l_last) < kMaxRange;
+            const float lref = l_last;
+            wv[lane] = lane >= row0 ? __expf(sl[lane] - lref) : 0.f;
+            wv[lane + 64] = lane + 64 >= row0 ? __expf(sl[lane + 64] - lref) : 0.f;
+            if (lane < 32) wu[lane] = __expf(fminf(lref - sl[row0 + lane], 0.f));
+            __syncthreads();
+            if (hh + 1 < a.hps) issue_tiles(h + 1, buf ^ 1);
+            const T* cS = tiles + buf * TILES;
+            const T* cP = cS + P * N;
+            const T* cY = cP + P * N;
+            const T* cX = cY + kQ * P;
+
+            const float off_fast = __expf(Lam - lref);
+            auto off_scale = [&](int v) -> float { return fast ? off_fast : __expf(Lam - sl[row0 + acc_row(lane, v)]); };
+            auto fin_scale = [&](int v) -> float { return fast ? wu[acc_row(lane, v)] : 1.f; };
+            // sum over this wave's channels of  t[row][p] * Z[row][p]  for its 16 accumulator rows (Z row-major tile, read
+            // at the accumulator positions by transpose reads); returns one row total per lane pair (see half_wave_reduce16)
+            auto row_dot = [&](const floatx16 (&t)[1][BN], const T* Z, float (&out)[16]) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float s4[4] = {0.f, 0.f, 0.f, 0.f};
+                    const int tok = row0 + 8 * q + 4 * half + tr_row;
+#pragma unroll
+                    for (int j = 0; j < BN; ++j) {
+                        const int col = j * 32 + tr_col;
+                        const tvec4 zv = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                            (M2_LDS tvec4*)(Z + (tok * SPR_X + ((col >> 3) ^ swz_x(tok))) * 8 + (col & 7)));
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) s4[e] += t[0][j][4 * q + e] * to_f32(zv[e]);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) out[4 * q + e] = s4[e];
+                }
+            };
+
+            // ---- dl_c: (C rows x S_prev) . dy, row scale e^{l_i}
+            {
+                floatx16 yo[1][BN];
+                acc_zero(yo);
+#pragma unroll
+                for (int ks = 0; ks < KSN; ++ks) {
+#pragma unroll
+                    for (int j = 0; j < BN; ++j) {
+                        const int row = j * 32 + r;
+                        const Frag<T> bf = load_frag(cP + (row * SPR_S + ((ks * 2 + half) ^ swz_s<SPR_S>(row))) * 8);
+                        mma_frag(yo[0][j], ks < KCR ? foC[ks < KCR ? ks : 0] : load_frag(sFCw + r * LDC + (ks - KCR) * 16 + half * 8), bf);
+                    }
+                }
+                float dv[16];
+                row_dot(yo, cY, dv);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = row0 + acc_row(lane, v);
+                    dv[v] *= row < valid ? __expf(sl[row]) : 0.f;
+                }
+                int ri;
+                const float tot = half_wave_reduce16(dv, &ri);
+                if ((lane & 1) == 0) a.dlc[bhc * kQ + row0 + acc_row(lane, ri)] = tot;
+            }
+
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- state part of dxd: B rows (registers) x dS (LDS, natural layout)
+            floatx16 acc[1][BN];
+            acc_zero(acc);
+#pragma unroll
+            for (int ks = 0; ks < KSN; ++ks) {
+#pragma unroll
+                for (int j = 0; j < BN; ++j) {
+                    const int row = j * 32 + r;
+                    const Frag<T> bf = load_frag(cS + (row * SPR_S + ((ks * 2 + half) ^ swz_s<SPR_S>(row))) * 8);
+                    mma_frag(acc[0][j], foB[ks], bf);
+                }
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float os = off_scale(v);
+#pragma unroll
+                for (int j = 0; j < BN; ++j) acc[0][j][v] *= os;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- rb_j = dt_j sum_p x[j][p] * (state part, final scale applied)
+            {
+                float rv[16];
+                row_dot(acc, cX, rv);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) rv[v] *= fin_scale(v);
+                int ri;
+                const float tot = half_wave_reduce16(rv, &ri);
+                const int row = row0 + acc_row(lane, ri);
+                if ((lane & 1) == 0) a.rbp[bhc * kQ + row] = tot * sd[row];
+            }
+
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- diagonal part: transposed causal C B^T fragment scaled along k = i; dy through transpose reads
+            const int jrow = row0 + r;
+            const float l_row = sl[jrow];
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                if (ks < 2 * rbk) continue;
+                float f[8];
+                if (fast) {
+                    const floatx4 fa = *reinterpret_cast<const floatx4*>(wv + ks * 16 + half * 8);
+                    const floatx4 fb = *reinterpret_cast<const floatx4*>(wv + ks * 16 + half * 8 + 4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) { f[e] = fa[e]; f[4 + e] = fb[e]; }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int k = ks * 16 + half * 8 + e;
+                        f[e] = (k >= jrow) ? __expf(sl[k] - l_row) : 0.f;
+                    }
+                }
+                keep_packed(fd[ks]);
+                keep_packed(fd[ks]);
+            const Frag<T> af = scale_frag(fd[ks], f);
+#pragma unroll
+                for (int j = 0; j < BN; ++j) {
+                    const int col = j * 32 + tr_col;
+                    const int ta = ks * 16 + 8 * half + tr_row, tb = ta + 4;
+                    const tvec4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                        (M2_LDS tvec4*)(cY + (ta * SPR_X + ((col >> 3) ^ swz_x(ta))) * 8 + (col & 7)));
+                    const tvec4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                        (M2_LDS tvec4*)(cY + (tb * SPR_X + ((col >> 3) ^ swz_x(tb))) * 8 + (col & 7)));
+                    Frag<T> bf;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) { bf.v[e] = lo[e]; bf.v[4 + e] = hi[e]; }
+                    mma_frag(acc[0][j], af, bf);
+                }
+            }
+
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- epilogue, 8 token rows at a time: fp32 through the wave-private tile, then row-wise
+            constexpr int LPR = P / 8;               // lanes per output row
+            constexpr int RPP = 64 / LPR;            // rows per pass
+            static_assert(RPP <= 8 && 8 % RPP == 0, "row passes");
+            T* dXp = static_cast<T*>(a.dx) + b * a.dx_sb + t0 * a.dx_sl + h * a.dx_sh;
+            float dD_loc = 0.f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+#pragma unroll
+                for (int j = 0; j < BN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) sYw[(4 * half + e) * P + j * 32 + r] = acc[0][j][4 * q + e] * fin_scale(4 * q + e);
+                wave_lds_sync();
+#pragma unroll
+                for (int ps = 0; ps < 8 / RPP; ++ps) {
+                    const int rl = ps * RPP + lane / LPR, cv = lane % LPR;
+                    const int tok = row0 + 8 * q + rl;
+                    const floatx4 ya = *reinterpret_cast<const floatx4*>(sYw + rl * P + cv * 8);
+                    const floatx4 yb = *reinterpret_cast<const floatx4*>(sYw + rl * P + cv * 8 + 4);
+                    const int slot = cv ^ swz_x(tok);
+                    const uint4 xr = *reinterpret_cast<const uint4*>(cX + (tok * SPR_X + slot) * 8);
+                    const uint4 gr = *reinterpret_cast<const uint4*>(cY + (tok * SPR_X + slot) * 8);
+                    const T* xe = reinterpret_cast<const T*>(&xr);
+                    const T* ge = reinterpret_cast<const T*>(&gr);
+                    const float dtt = sd[tok];
+                    uint4 ov;
+                    T* oe = reinterpret_cast<T*>(&ov);
+                    float dir = 0.f, dd = 0.f;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float dxd = e < 4 ? ya[e] : yb[e - 4];
+                        const float x_ = to_f32(xe[e]), gy = to_f32(ge[e]);
+                        oe[e] = from_f32<T>(dtt * dxd + Dh * gy);
+                        dir += dxd * x_;
+                        dd += gy * x_;
+                    }
+                    if (tok < valid) {
+                        *reinterpret_cast<uint4*>(dXp + (int64_t)tok * a.dx_sl + cv * 8) = ov;
+                        dD_loc += dd;
+                    }
+#pragma unroll
+                    for (int m = 1; m < LPR; m <<= 1) dir += __shfl_xor(dir, m, 64);      // the LPR lanes that share the row
+                    if (cv == 0) a.dirp[bhc * kQ + tok] = dir;
+                }
+                wave_lds_sync();
+            }
+            dD_loc = warp_sum(dD_loc);
+            if (lane == 0) { a.dDp8[bhc * 8 + wave] = dD_loc; a.dDp8[bhc * 8 + wave + 4] = 0.f; }
+        }
+    } else {
+        // =============================================================== role B: state parts of dB and dC
+        floatx16 accB[1][NBN], accC[1][NBN];
+        acc_zero(accB);
+        acc_zero(accC);
+        for (int64_t hh = 0; hh < a.hps; ++hh) {
+            const int64_t h = h_first + hh;
+            const int buf = (int)(hh & 1);
+            wait_vmem_all();
+            const float* sl = sLD + buf * 2 * kQ;
+            const float* sd = sl + kQ;
+            __syncthreads();
+            if (hh + 1 < a.hps) issue_tiles(h + 1, buf ^ 1);
+            const T* cS = tiles + buf * TILES;
+            const T* cP = cS + P * N;
+            const T* cY = cP + P * N;
+            const T* cX = cY + kQ * P;
+            const int tok = row0 + r;
+            // t[n-block] = sum_p Rows[tok][p] * St[p][n]: rows as they lie (A operand), the state tile through transpose reads
+            auto rows_times_state = [&](const T* Rows, const T* St, bool side_b, floatx16 (&accum)[1][NBN]) {
+                // row scales of this lane's 16 accumulator rows: dt_j e^{Lam - l_j} (dB side) or e^{l_i} (dC side; 0 past the end)
+                float ws[16];
+                {
+                    const float Lam = sl[kQ - 1];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int row = row0 + acc_row(lane, v);
+                        const float lr = sl[row];
+                        ws[v] = side_b ? sd[row] * __expf(Lam - lr) : (row < valid ? __expf(lr) : 0.f);
+                    }
+                }
+#pragma unroll
+                for (int jn = 0; jn < NBN; ++jn) {
+                    floatx16 t = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                    const int col = jn * 32 + tr_col;
+#pragma unroll
+                    for (int ks = 0; ks < KSP; ++ks) {
+                        const int pa = ks * 16 + 8 * half + tr_row, pb = pa + 4;
+                        const tvec4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                            (M2_LDS tvec4*)(St + (pa * SPR_S + ((col >> 3) ^ swz_s<SPR_S>(pa))) * 8 + (col & 7)));
+                        const tvec4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                            (M2_LDS tvec4*)(St + (pb * SPR_S + ((col >> 3) ^ swz_s<SPR_S>(pb))) * 8 + (col & 7)));
+                        Frag<T> bf;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) { bf.v[e] = lo[e]; bf.v[4 + e] = hi[e]; }
+                        mma_frag(t, load_frag(Rows + (tok * SPR_X + ((ks * 2 + half) ^ swz_x(tok))) * 8), bf);
+                    }
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) accum[0][jn][v] += t[v] * ws[v];
+                    __builtin_amdgcn_sched_barrier(0);      // keep the next block's operand reads from being hoisted up here
+                }
+            };
+            rows_times_state(cX, cS, true, accB);
+            rows_times_state(cY, cP, false, accC);
+        }
+        const int64_t part = (((b * a.nchunks + c) * a.ngroups + g) * a.nslices + slice) * (int64_t)(kQ * N);
+#pragma unroll
+        for (int jn = 0; jn < NBN; ++jn)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int64_t o = part + (row0 + acc_row(lane, v)) * N + jn * 32 + r;
+                a.dBp[o] = accB[0][jn][v];
+                a.dCp[o] = accC[0][jn][v];
+            }
+    }
+}
+
+// Per (batch, head, chunk): da_t = sum_{i>=t} (dl_diag_i + dl_c_i) + sum_{j<t} rb_j + dlam,  ddt_t = A da_t + dir_t,
+// dA partial = sum_t da_t dt_t, dD partial = sum of the per-wave partials.  One wave per (b, h, c), four per
+// workgroup; lanes hold the tokens in reverse order (127 - lane, 63 - lane), so the suffix over tokens is an inclusive
+// prefix over lanes and the exclusive prefix over tokens an exclusive suffix over lanes.
+template <typename T>
+__global__ void __launch_bounds__(256)
+da_kernel(const float* __restrict__ ldtab, const float* __restrict__ A,
+          const float* __restrict__ dl_diag, const float* __restrict__ dl_c, const float* __restrict__ dlam,
+          const float* __restrict__ dirp, const float* __restrict__ rbp, const float* __restrict__ dDp8,
+          void* __restrict__ ddt, int dt_f32, int64_t ddt_sb, int64_t ddt_sl, float* __restrict__ dAp, float* __restrict__ dDp,
+          int64_t seqlen, int64_t nheads, int64_t nchunks, int64_t total) {
+    const int lane = threadIdx.x & 63;
+    const int64_t bhc = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (bhc >= total) return;
+    const int64_t c = bhc % nchunks, h = (bhc / nchunks) % nheads, b = bhc / (nchunks * nheads);
+    const int64_t t0 = c * kQ;
+    const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
+    const int ta = kQ - 1 - lane, tb = 63 - lane;
+    const float Ah = A[h];
+    float xa = dl_diag[bhc * kQ + ta] + dl_c[bhc * kQ + ta];
+    float xb = dl_diag[bhc * kQ + tb] + dl_c[bhc * kQ + tb];
+    const float ra = rbp[bhc * kQ + ta], rbv = rbp[bhc * kQ + tb];
+    const float dira = dirp[bhc * kQ + ta], dirb = dirp[bhc * kQ + tb];
+    const float dta = ldtab[bhc * 2 * kQ + kQ + ta], dtb = ldtab[bhc * 2 * kQ + kQ + tb];     // 0 past the end of the sequence
+    float dlm = 0.f;
+#pragma unroll
+    for (int sp = 0; sp < kScanSplit; ++sp) dlm += dlam[bhc * kScanSplit + sp];
+    float ya = ra, yb = rbv;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const float na = __shfl_up(xa, o, 64), nb = __shfl_up(xb, o, 64);
+        const float ma = __shfl_down(ya, o, 64), mb = __shfl_down(yb, o, 64);
+        if (lane >= o) { xa += na; xb += nb; }
+        if (lane + o < 64) { ya += ma; yb += mb; }
+    }
+    xb += __shfl(xa, 63, 64);
+    xa += (ya - ra) + __shfl(yb, 0, 64);
+    xb += yb - rbv;
+    const float da_a = xa + dlm, da_b = xb + dlm;
+    float dAl = 0.f;
+    if (ta < valid) {
+        const float val = Ah * da_a + dira;
+        const int64_t oo = b * ddt_sb + (t0 + ta) * ddt_sl + h;
+        if (dt_f32) static_cast<float*>(ddt)[oo] = val; else static_cast<T*>(ddt)[oo] = from_f32<T>(val);
+        dAl += da_a * dta;
+    }
+    if (tb < valid) {
+        const float val = Ah * da_b + dirb;
+        const int64_t oo = b * ddt_sb + (t0 + tb) * ddt_sl + h;
+        if (dt_f32) static_cast<float*>(ddt)[oo] = val; else static_cast<T*>(ddt)[oo] = from_f32<T>(val);
+        dAl += da_b * dtb;
+    }
+    dAl = warp_sum(dAl);
+    if (lane == 0) {
+        dAp[bhc] = dAl;
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) s += dDp8[bhc * 8 + w];
+        dDp[bhc] = s;
+    }
+}
+
+}  // namespace m2

@@ -48,20 +48,26 @@ dg16_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
     const int rb = wave >> 1, cb0 = (wave & 1) * 2;
     const bool active = cb0 <= rb;
 
+    const uint32_t wave_u = uniform(wave), lds_T = uniform(lds_addr_of(tiles)), lds_LD = uniform(lds_addr_of(sLD));
+    uint32_t offY[NX], offX[NX];      // per-lane source byte offsets (head-independent)
+#pragma unroll
+    for (int it = 0; it < NX; ++it) {
+        const int s = (wave * NX + it) * 64 + lane;
+        const int row = s / SPR, cs = (s % SPR) ^ (row & (SPR - 1));
+        const int grow = row < valid ? row : valid - 1;     // rows past the end: finite stand-ins, masked below
+        offY[it] = (uint32_t)(grow * dYsl + cs * 8) * 2u;
+        offX[it] = (uint32_t)(grow * Xsl + cs * 8) * 2u;
+    }
     auto issue_tiles = [&](int64_t h, int buf) {
-        T* dA_ = tiles + buf * 2 * TILE;
-        T* dT_ = dA_ + TILE;
         const T* gy = dY + b * dYsb + t0 * dYsl + h * dYsh;
         const T* gx = X + b * Xsb + t0 * Xsl + h * Xsh;
+        const uint32_t dst = lds_T + (uint32_t)(buf * 2 * TILE * 2);
 #pragma unroll
         for (int it = 0; it < NX; ++it) {
-            const int s0 = (wave * NX + it) * 64, s = s0 + lane;
-            const int row = s / SPR, cs = (s % SPR) ^ (row & (SPR - 1));
-            const int grow = row < valid ? row : valid - 1;     // rows past the end: finite stand-ins, masked below
-            async_copy16(gy + (int64_t)grow * dYsl + cs * 8, dA_ + s0 * 8);
-            async_copy16(gx + (int64_t)grow * Xsl + cs * 8, dT_ + s0 * 8);
+            async_copy16(gy, offY[it], dst + (wave_u * NX + it) * 1024u);
+            async_copy16(gx, offX[it], dst + (uint32_t)(TILE * 2) + (wave_u * NX + it) * 1024u);
         }
-        async_copy_ldtab(ldtab, (b * nheads + h) * nchunks + c, sLD + buf * 2 * kQ);
+        async_copy_ldtab(ldtab, (b * nheads + h) * nchunks + c, lds_LD + (uint32_t)(buf * 2 * kQ * 4));
     };
     const int64_t h_first = g * hpg + slice * hps;
 #pragma unroll

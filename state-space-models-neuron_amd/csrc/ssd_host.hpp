@@ -2,7 +2,7 @@
 #pragma once
 #include "ssd_kernels.hpp"
 #include "ssd_diag.hpp"
-#include "ssd_dx.hpp"
+#include "ssd_bwd_main.hpp"
 #include "ssd_dg.hpp"
 
 namespace m2 {
@@ -91,6 +91,10 @@ inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd, bool
         ssd_slicing(p, kWgsDg, &w.ns_g, &w.hps_g);
         ssd_slicing(p, kWgsOffC, &w.ns_c, &w.hps_c);
         ssd_slicing(p, kWgsOffB, &w.ns_b, &w.hps_b);
+        if (p->dtype != M2_F32 && p->headdim == 64) {       // the main backward kernel produces both state parts there
+            ssd_slicing(p, kWgsDx, &w.ns_b, &w.hps_b);
+            w.ns_c = w.ns_b; w.hps_c = w.hps_b;
+        }
         w.dprev = take(tiles * esz);
         w.dlam = reinterpret_cast<float*>(take(bhc * 4 * kScanSplit));
         w.dAp = reinterpret_cast<float*>(take(bhc * 4));

@@ -49,22 +49,25 @@ __device__ __forceinline__ void wait_vmem_keep(int groups) {
     asm volatile("" ::: "memory");
 }
 
-// Asynchronous 16-byte-per-lane copy global -> LDS: lane i's 16 bytes land at lds_base + 16 i (lds_base wave-uniform).
+// Asynchronous 16-byte-per-lane copy global -> LDS: lane i reads 16 bytes at  gbase + voff_i  (gbase wave-uniform, voff a
+// per-lane BYTE offset) and they land at LDS byte address  lds_addr + 16 i  (lds_addr wave-uniform).
 // Written as inline assembly on purpose: for the compiler's own direct-to-LDS builtin the wait-count pass
 // makes every later LDS store (and transpose read) wait for ALL outstanding vector-memory operations, which
 // serialises exactly the copy/compute overlap this is for.  Completion is awaited explicitly (wait_vmem_all) before
 // the barrier that publishes the tile; operations the compiler does not know about can only make its own
 // vmcnt waits more conservative, never too short (vmcnt retires in order).
-__device__ __forceinline__ void async_copy16(const void* gsrc, void* lds_base) {
-    const uint32_t l = __builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(M2_LDS void*)lds_base);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gsrc), "s"(l) : "memory", "m0");
+__device__ __forceinline__ void async_copy16(const void* gbase, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(gbase), "s"(lds_addr) : "memory");
 }
+// LDS byte address of a pointer into shared memory / a value the compiler may keep in a scalar register
+__device__ __forceinline__ uint32_t lds_addr_of(const void* p) { return (uint32_t)(uintptr_t)(M2_LDS const void*)p; }
+__device__ __forceinline__ uint32_t uniform(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 
 // The [ l | dt ] table of one (batch, head, chunk): 2 kQ floats = 64 lanes x 16 bytes, one wave-wide copy.  Every
 // wave of the workgroup issues it (same source, same destination, same data), so each wave may read the table as
 // soon as ITS OWN copies have landed, and all waves issue the same number of vector-memory operations per head.
-__device__ __forceinline__ void async_copy_ldtab(const float* __restrict__ ldtab, int64_t bhc, float* lds_tab) {
-    async_copy16(ldtab + bhc * (2 * kQ) + (threadIdx.x & 63) * 4, lds_tab);
+__device__ __forceinline__ void async_copy_ldtab(const float* __restrict__ ldtab, int64_t bhc, uint32_t lds_addr) {
+    async_copy16(ldtab + bhc * (2 * kQ), (threadIdx.x & 63) * 16u, lds_addr);
 }
 
 // 16-byte slot s of row `row` lives at slot (s ^ swz) of that row
@@ -103,29 +106,31 @@ ssd_y16_kernel(const DiagArgs a) {
     float* wu = wv + kQ;          // [32]: rows row0 .. row0 + 31
     float* sYw = sY + wave * 8 * P;
 
-    // ---- asynchronous tile copy of one head into buffer `buf`
+    // ---- asynchronous tile copy of one head into buffer `buf`; the per-lane source offsets do not depend on the head
+    const uint32_t wave_u = uniform(wave), lds_S = uniform(lds_addr_of(sS)), lds_X = uniform(lds_addr_of(sX)), lds_LD = uniform(lds_addr_of(sLD));
+    uint32_t offS[NS], offX[NX];
+#pragma unroll
+    for (int it = 0; it < NS; ++it) {
+        const int s = (wave * NS + it) * 64 + lane;
+        const int row = s / SPR_S, cs = (s % SPR_S) ^ swz_s<SPR_S>(row);
+        offS[it] = (uint32_t)(row * N + cs * 8) * 2u;
+    }
+#pragma unroll
+    for (int it = 0; it < NX; ++it) {
+        const int s = (wave * NX + it) * 64 + lane;
+        const int row = s / SPR_X, cs = (s % SPR_X) ^ swz_x(row);
+        // rows past the end of the sequence re-read the last valid row: their dt is 0, so they only ever meet zeros
+        const int grow = row < valid ? row : valid - 1;
+        offX[it] = (uint32_t)(grow * a.Z_sl + cs * 8) * 2u;
+    }
     auto issue_tiles = [&](int64_t h, int buf) {
         const T* Sp = static_cast<const T*>(a.S) + ((b * a.nchunks + c) * a.nheads + h) * (int64_t)(P * N);
-        T* dS = sS + buf * (P * N);
 #pragma unroll
-        for (int it = 0; it < NS; ++it) {
-            const int s0 = (wave * NS + it) * 64;              // first slot of this wave-wide load
-            const int s = s0 + lane;
-            const int row = s / SPR_S, cs = (s % SPR_S) ^ swz_s<SPR_S>(row);
-            async_copy16(Sp + row * N + cs * 8, dS + s0 * 8);
-        }
+        for (int it = 0; it < NS; ++it) async_copy16(Sp, offS[it], lds_S + (uint32_t)(buf * (P * N) * 2) + (wave_u * NS + it) * 1024u);
         const T* Xp = static_cast<const T*>(a.Z) + b * a.Z_sb + t0 * a.Z_sl + h * a.Z_sh;
-        T* dX = sX + buf * (kQ * P);
 #pragma unroll
-        for (int it = 0; it < NX; ++it) {
-            const int s0 = (wave * NX + it) * 64;
-            const int s = s0 + lane;
-            const int row = s / SPR_X, cs = (s % SPR_X) ^ swz_x(row);
-            // rows past the end of the sequence re-read the last valid row: their dt is 0, so they only ever meet zeros
-            const int grow = row < valid ? row : valid - 1;
-            async_copy16(Xp + (int64_t)grow * a.Z_sl + cs * 8, dX + s0 * 8);
-        }
-        async_copy_ldtab(a.ldtab, (b * a.nheads + h) * a.nchunks + c, sLD + buf * 2 * kQ);
+        for (int it = 0; it < NX; ++it) async_copy16(Xp, offX[it], lds_X + (uint32_t)(buf * (kQ * P) * 2) + (wave_u * NX + it) * 1024u);
+        async_copy_ldtab(a.ldtab, (b * a.nheads + h) * a.nchunks + c, lds_LD + (uint32_t)(buf * 2 * kQ * 4));
     };
 
     const int64_t h_first = g * hpg + slice * a.hps;
@@ -216,6 +221,7 @@ ssd_y16_kernel(const DiagArgs a) {
                     f[e] = (k <= jrow) ? __expf(l_row - sl[k]) * sd[k] : 0.f;
                 }
             }
+            keep_packed(fd[ks]);
             const Frag<T> af = scale_frag(fd[ks], f);
 #pragma unroll
             for (int j = 0; j < BN; ++j) {
