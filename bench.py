@@ -25,6 +25,11 @@ sys.path.insert(0, os.path.join(ROOT, "state-space-models-neuron_amd"))
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0     # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0              # MI355X HBM3E
+# Measured HBM bytes per step (rocprofv3 FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, the factors the 1 GiB copy kernel
+# gives in the same runs; profiles/bench_all_workloads_kernels.md).  They describe the kernels as profiled, not this run.
+SSD_TRAFFIC_BYTES = 2.15e9
+CONV_TRAFFIC_BYTES = 460.7e6
+DECODE_TRAFFIC_BYTES = 64 * 689.3e6
 
 SSD_CFG = dict(b=4, l=2048, h=80, p=64, n=128, g=1)
 CONV_CFG = dict(b=4, l=2048, C=5376, k=4)
@@ -101,7 +106,7 @@ def bench_conv(steps, warmup):
     return dict(metric="conv1d+SiLU fwd+bwd tokens/s", value=tokens / (ms * 1e-3), unit="tokens/s", ms_per_step=ms, dtype="bf16",
                 config={"workload": "depthwise conv1d k=4 + SiLU fwd+bwd, b4 l2048 C5376, channels-last"},
                 roofline={"bound": "hbm", "achieved": bytes_ / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                          "frac": bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": CONV_TRAFFIC_BYTES,
                           "algorithmic_bytes_per_step": bytes_, "kernels": "conv_fwd_cl_kernel + conv_bwd_cl_kernel + conv_reduce_partials_kernel"})
 
 
@@ -130,7 +135,7 @@ def bench_decode(steps, warmup):
                 us_per_sequence_token=ms * 1e3 / cfg["b"], ms_per_step=ms, wall_ms_per_step=wall_ms, dtype="f32 state / bf16 activations",
                 config={"workload": "decode step, 64 layers x (b128, h80, p64, n128, C5376, W3), states in place"},
                 roofline={"bound": "hbm", "achieved": bytes_ / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                          "frac": bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": DECODE_TRAFFIC_BYTES,
                           "algorithmic_bytes_per_step": bytes_, "kernels": "decode_conv_kernel + decode_ssm_kernel, 64 launches each"})
 
 
@@ -209,7 +214,7 @@ def main():
             "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "Mamba-2 2.7B-shaped SSD chunked scan fwd+bwd: b4 l2048 h80 p64 n128 g1 chunk128, bf16 I/O, fp32 state"},
             "roofline": {"bound": "mfma", "achieved": r["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": r["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                         "frac": r["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": SSD_TRAFFIC_BYTES,
                          "algorithmic_flops_per_step": r["flops"], "event_ms_avg": r["ms_event_avg"],
                          "event_ms_min": r["ms_event_min"],
                          "kernels": "all launches of m2_ssd_fwd + m2_ssd_bwd (one step), HIP events on the launch stream"},
