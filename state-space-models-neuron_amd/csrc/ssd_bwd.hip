@@ -63,7 +63,7 @@ dg_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
     T* sG = sT + kQ * LDP;                                 // G  [kQ][LDQ]  (blocks above the diagonal are never read)
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int r = lane & 31, half = lane >> 5;
+    const int r = lane & 31;
     const int64_t c = blockIdx.x, b = blockIdx.z;
     const int64_t g = blockIdx.y / nslices, slice = blockIdx.y % nslices;
     const int64_t hpg = nheads / ngroups;

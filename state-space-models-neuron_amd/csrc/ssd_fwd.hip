@@ -5,10 +5,11 @@
 // that every (batch, head, chunk) tile is an independent workgroup (thousands of them for 256 CUs)
 // and only a cheap elementwise recurrence is sequential in the chunk index:
 //
+//   0. ld_table_kernel     l = cumsum(A dt) per chunk        per (b, head, chunk)    scan
 //   1. cb_kernel           G = C B^T                         per (b, chunk, group)   MFMA
 //   2. chunk_state_kernel  local state B^T (decay o dt o X)  per (b, chunk, head)    MFMA
 //   3. state_scan_kernel   S_prev(c), final state            per (b, head)           fp32 FMA
-//   4. chunk_scan_kernel   Y = (L o G)(dt o X) + e^l C S_prev + D X   per (b, chunk, head)   MFMA
+//   4. ssd_y16_kernel (16-bit) / diag_off_kernel<false>      Y = (L o G)(dt o X) + e^l C S_prev + D X   MFMA
 //
 // Extensions over the reference kernel: optional initial state, final-state output, any batch,
 // ragged sequence length (tokens past the end behave as dt = 0 and are never written).
@@ -17,98 +18,6 @@
 
 namespace m2 {
 namespace {
-
-// ------------------------------------------------------------------------------------------
-// grid (nchunks, nheads, batch), 256 threads (4 waves; wave w owns output rows 32w..32w+31).
-template <typename T, int P, int N>
-__global__ void __launch_bounds__(256)
-chunk_scan_kernel(const T* __restrict__ X, const void* __restrict__ dt, int dt_f32, const float* __restrict__ A,
-                  const T* __restrict__ Cm, const float* __restrict__ D, const float* __restrict__ G,
-                  const T* __restrict__ Sprev, T* __restrict__ Y,
-                  int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks,
-                  int64_t Xsb, int64_t Xsl, int64_t Xsh, int64_t dtsb, int64_t dtsl,
-                  int64_t Csb, int64_t Csl, int64_t Csg, int64_t Ysb, int64_t Ysl, int64_t Ysh) {
-    constexpr int LDN = lds_ld<T>(N);      // tiles with N (state) columns
-    constexpr int LDQ = lds_ld<T>(kQ);     // tiles with Q (token) columns
-    constexpr int BN = P / 32;
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    float* s_l = reinterpret_cast<float*>(smem_raw);
-    float* s_dt = s_l + kQ;
-    float* s_tmp = s_dt + kQ;                       // 4 floats
-    T* buf = reinterpret_cast<T*>(s_tmp + 4);
-    // phase 1: sC [kQ][LDN], sS [P][LDN];   phase 2: sM [kQ][LDQ], sXt [P][LDQ]   (same memory)
-    T* sC = buf;
-    T* sS = buf + kQ * LDN;
-    T* sM = buf;
-    T* sXt = buf + kQ * LDQ;
-
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int64_t c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    const int64_t g = h / (nheads / ngroups);
-    const int64_t t0 = c * kQ;
-    const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
-
-    chunk_cumsum_any<T>(dt, dt_f32, b * dtsb + t0 * dtsl + h, dtsl, valid, A[h], s_l, s_dt, s_tmp, tid);
-
-    // ---- phase 1: off-diagonal term  acc[t][p] = e^{l_t} * sum_n C[t][n] S_prev[p][n]
-    const int64_t tile = ((b * nchunks + c) * nheads + h) * (int64_t)(P * N);
-    stage_rows<T, kQ, N, 256, false>(sC, LDN, Cm + b * Csb + t0 * Csl + g * Csg, Csl, valid, nullptr, tid);
-    stage_rows<T, P, N, 256, false>(sS, LDN, Sprev + tile, N, P, nullptr, tid);
-    __syncthreads();
-    floatx16 acc[1][BN];
-    acc_zero(acc);
-    wave_mma<1, BN>(acc, sC + wave * 32 * LDN, LDN, sS, LDN, 0, N);
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const float e = __expf(s_l[wave * 32 + acc_row(lane, v)]);
-#pragma unroll
-        for (int j = 0; j < BN; ++j) acc[0][j][v] *= e;
-    }
-    __syncthreads();     // everyone done reading sC / sS
-
-    // ---- phase 2: diagonal term  acc[t][p] += sum_{s<=t} (e^{l_t-l_s} dt_s G[t][s]) x[s][p]
-    const float* Gp = G + ((b * nchunks + c) * ngroups + g) * (int64_t)(kQ * kQ);
-    for (int e = tid; e < kQ * (kQ / 4); e += 256) {
-        const int t = e / (kQ / 4), s4 = (e % (kQ / 4)) * 4;
-        if ((s4 >> 5) > (t >> 5)) continue;           // 32x32 block above the diagonal: never read
-        const floatx4 g4 = *reinterpret_cast<const floatx4*>(Gp + t * kQ + s4);
-        const float lt = s_l[t];
-        T o[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int s = s4 + q;
-            const float m = (s <= t) ? __expf(lt - s_l[s]) * s_dt[s] * g4[q] : 0.f;
-            o[q] = from_f32<T>(m);
-        }
-        if (sizeof(T) == 2) *reinterpret_cast<uint2*>(sM + t * LDQ + s4) = *reinterpret_cast<const uint2*>(o);
-        else *reinterpret_cast<uint4*>(sM + t * LDQ + s4) = *reinterpret_cast<const uint4*>(o);
-    }
-    const T* Xp = X + b * Xsb + t0 * Xsl + h * Xsh;
-    stage_transposed<T, kQ, P, 256, false>(sXt, LDQ, Xp, Xsl, valid, nullptr, tid);
-    __syncthreads();
-    wave_mma<1, BN>(acc, sM + wave * 32 * LDQ, LDQ, sXt, LDQ, 0, (wave + 1) * 32);
-
-    // ---- epilogue: + D x, store
-    const float Dh = D ? D[h] : 0.f;
-    T* Yp = Y + b * Ysb + t0 * Ysl + h * Ysh;
-#pragma unroll
-    for (int j = 0; j < BN; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int row = wave * 32 + acc_row(lane, v);
-            const int col = j * 32 + acc_col(lane);
-            if (row < valid) {
-                const float xv = to_f32(sXt[col * LDQ + row]);
-                Yp[(int64_t)row * Ysl + col] = from_f32<T>(acc[0][j][v] + Dh * xv);
-            }
-        }
-}
-
-template <typename T, int P, int N>
-size_t scan_smem() {
-    const size_t a = (size_t)(kQ + P) * lds_ld<T>(N), b = (size_t)(kQ + P) * lds_ld<T>(kQ);
-    return (2 * kQ + 4) * sizeof(float) + (a > b ? a : b) * sizeof(T);
-}
 
 // zero-length sequence: y is empty; the final state is the initial state (or zero)
 __global__ void copy_or_zero_kernel(const float* __restrict__ src, float* __restrict__ dst, int64_t n) {

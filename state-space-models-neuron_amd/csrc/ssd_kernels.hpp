@@ -23,9 +23,6 @@
 
 namespace m2 {
 
-struct SsdDims {
-    int64_t batch, seqlen, nheads, ngroups, nchunks;
-};
 
 // ------------------------------------------------------------------------------------------
 // Per (batch, chunk, group): G = C B^T and the head-independent operand tiles every other kernel reuses.
