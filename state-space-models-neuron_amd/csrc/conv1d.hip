@@ -37,8 +37,40 @@ constexpr int kMaxK = 8;
 #endif
 constexpr int kTL = M2_CONV_TL;      // tokens per thread in the fast path
 constexpr int kUNR = M2_CONV_UNR;    // tokens whose loads are in flight together
-constexpr int kCVT = 32;       // channel vectors per block (x dimension)
-constexpr int kSEG = 8;        // token segments per block (y dimension)
+#ifndef M2_CONV_CVT
+#define M2_CONV_CVT 32
+#endif
+#ifndef M2_CONV_SEG
+#define M2_CONV_SEG 8
+#endif
+#ifndef M2_CONV_NT
+#define M2_CONV_NT 1
+#endif
+constexpr int kCVT = M2_CONV_CVT;    // channel vectors per block (x dimension)
+constexpr int kSEG = M2_CONV_SEG;    // token segments per block (y dimension)
+
+// streaming loads/stores of the activations (optionally non-temporal: nothing is re-read soon enough to be worth caching)
+template <int BYTES> struct StreamVec;
+template <> struct StreamVec<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
+template <> struct StreamVec<8> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
+template <> struct StreamVec<4> { typedef uint32_t type; };
+template <typename T, int V>
+__device__ __forceinline__ RawVec<T, V> ld_stream(const T* __restrict__ p) {
+    using S = typename StreamVec<V * (int)sizeof(T)>::type;
+    RawVec<T, V> r;
+    const S v = M2_CONV_NT ? __builtin_nontemporal_load(reinterpret_cast<const S*>(p)) : *reinterpret_cast<const S*>(p);
+    *reinterpret_cast<S*>(&r) = v;
+    return r;
+}
+template <typename T, int V>
+__device__ __forceinline__ void st_stream(T* __restrict__ p, const float (&in)[V]) {
+    using S = typename StreamVec<V * (int)sizeof(T)>::type;
+    S raw;
+    T* e = reinterpret_cast<T*>(&raw);
+#pragma unroll
+    for (int i = 0; i < V; ++i) e[i] = from_f32<T>(in[i]);
+    if (M2_CONV_NT) __builtin_nontemporal_store(raw, reinterpret_cast<S*>(p)); else *reinterpret_cast<S*>(p) = raw;
+}
 
 __device__ __forceinline__ float ld_param(const void* p, int pd, int64_t i) {
     return pd == M2_F32 ? reinterpret_cast<const float*>(p)[i] : to_f32(reinterpret_cast<const bf16_t*>(p)[i]);
@@ -83,14 +115,14 @@ conv_fwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const vo
     RawVec<T, V> nxt[kUNR];
 #pragma unroll
     for (int u = 0; u < kUNR; ++u)
-        if (t0 + u < t1) nxt[u] = loadv_raw<T, V>(xp + (t0 + u) * xsl);
+        if (t0 + u < t1) nxt[u] = ld_stream<T, V>(xp + (t0 + u) * xsl);
     for (int64_t tg = t0; tg < t1; tg += kUNR) {
         RawVec<T, V> raw[kUNR];
 #pragma unroll
         for (int u = 0; u < kUNR; ++u) raw[u] = nxt[u];
 #pragma unroll
         for (int u = 0; u < kUNR; ++u)
-            if (tg + kUNR + u < t1) nxt[u] = loadv_raw<T, V>(xp + (tg + kUNR + u) * xsl);
+            if (tg + kUNR + u < t1) nxt[u] = ld_stream<T, V>(xp + (tg + kUNR + u) * xsl);
 #pragma unroll
         for (int u = 0; u < kUNR; ++u) {
             if (tg + u < t1) {
@@ -102,7 +134,7 @@ conv_fwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const vo
                     out[j] = act_f<ACT>(z);
                     h0[j] = h1[j]; h1[j] = h2[j]; h2[j] = cur[j];
                 }
-                storev<T, V>(yp + (tg + u) * ysl, out);
+                st_stream<T, V>(yp + (tg + u) * ysl, out);
             }
         }
     }
@@ -156,7 +188,7 @@ conv_bwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const vo
 #pragma unroll
         for (int u = 0; u < kUNR; ++u) {
             const int64_t t = t0 + u;
-            if (t < tend && t < l) { nx[u] = loadv_raw<T, V>(xp + t * xsl); ng[u] = loadv_raw<T, V>(gp + t * gsl); }
+            if (t < tend && t < l) { nx[u] = ld_stream<T, V>(xp + t * xsl); ng[u] = ld_stream<T, V>(gp + t * gsl); }
             else { nx[u] = RawVec<T, V>{}; ng[u] = RawVec<T, V>{}; }
         }
         for (int64_t tg = t0; tg < tend; tg += kUNR) {
@@ -166,7 +198,7 @@ conv_bwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const vo
 #pragma unroll
             for (int u = 0; u < kUNR; ++u) {
                 const int64_t t = tg + kUNR + u;
-                if (t < tend && t < l) { nx[u] = loadv_raw<T, V>(xp + t * xsl); ng[u] = loadv_raw<T, V>(gp + t * gsl); }
+                if (t < tend && t < l) { nx[u] = ld_stream<T, V>(xp + t * xsl); ng[u] = ld_stream<T, V>(gp + t * gsl); }
                 else { nx[u] = RawVec<T, V>{}; ng[u] = RawVec<T, V>{}; }
             }
 #pragma unroll
@@ -194,7 +226,7 @@ conv_bwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const vo
 #pragma unroll
                         for (int j = 0; j < V; ++j)
                             o[j] = wv[3][j] * g0[j] + wv[2][j] * g1[j] + wv[1][j] * g2[j] + wv[0][j] * g[j];
-                        storev<T, V>(dp + (t - 3) * dsl, o);
+                        st_stream<T, V>(dp + (t - 3) * dsl, o);
                     }
 #pragma unroll
                     for (int j = 0; j < V; ++j) {
