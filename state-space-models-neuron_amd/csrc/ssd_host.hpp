@@ -177,23 +177,27 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
             p->C_stride_b, p->C_stride_l, p->C_stride_g);
         if ((rc = check_launch("ssd cb_kernel"))) return rc;
     }
-    {
-        auto k = chunk_state_kernel<T, P, N, false>;
+    // per-chunk contributions in fp32 when an fp32 state leaves the call, otherwise in the operand type
+    auto states = [&](auto lt_tag) -> int {
+        using LT = decltype(lt_tag);
+        auto k = chunk_state_kernel<T, P, N, false, LT>;
         const size_t sm = state_smem<T, P, N>();
-        if ((rc = allow_smem(k, sm))) return rc;
+        int rc2;
+        if ((rc2 = allow_smem(k, sm))) return rc2;
         int64_t ns, hps;
         ssd_slicing(p, kWgsChunkState, &ns, &hps);
         M2_REQUIRE(p->ngroups * ns <= 65535, M2_ERR_SHAPE, "ssd: too many group slices");
         k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * ns), (unsigned)p->batch), 256, sm, st>>>(
-            x, w.ldtab, static_cast<const T*>(w.Bt), w.local, p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
+            x, w.ldtab, static_cast<const T*>(w.Bt), reinterpret_cast<LT*>(w.local), p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
             p->x_stride_b, p->x_stride_l, p->x_stride_h);
-        if ((rc = check_launch("ssd chunk_state_kernel"))) return rc;
-    }
-    {
-        state_scan_kernel<T, P * N, false><<<dim3((unsigned)p->nheads, (unsigned)p->batch, kScanSplit), 256, 0, st>>>(
-            w.local, w.lam, p->initial_state, static_cast<T*>(w.prev), final_out, nullptr, nullptr, p->nheads, nc);
-        if ((rc = check_launch("ssd state_scan_kernel"))) return rc;
-    }
+        if ((rc2 = check_launch("ssd chunk_state_kernel"))) return rc2;
+        state_scan_kernel<T, P * N, false, LT><<<dim3((unsigned)p->nheads, (unsigned)p->batch, kScanSplit), 256, 0, st>>>(
+            reinterpret_cast<const LT*>(w.local), w.lam, p->initial_state, static_cast<T*>(w.prev), final_out, nullptr, nullptr, p->nheads, nc);
+        return check_launch("ssd state_scan_kernel");
+    };
+    if (final_out) rc = states(float{});
+    else rc = states(T{});
+    if (rc) return rc;
     return M2_OK;
 }
 

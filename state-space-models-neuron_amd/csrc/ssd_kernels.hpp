@@ -126,13 +126,16 @@ ld_table_kernel(const void* __restrict__ dt, int dt_f32, const float* __restrict
 // Local chunk state.  grid (nchunks, ngroups * nslices, batch), 256 threads; a workgroup loops over `hps` heads.
 //   DSTATE == false:  out[p][n] = sum_j (dt_j e^{Lam-l_j}) x[j][p] * B[j][n]      (forward)
 //   DSTATE == true :  out[p][n] = sum_i e^{l_i} dy[i][p] * C[i][n]                (backward)
+// `out` is stored as LT: fp32, or -- for 16-bit operands when no fp32 state leaves the call (no final state / no
+// gradient of the initial state requested) -- the operand type, which halves the traffic of this kernel's output
+// and of the scan's input; the scan itself always accumulates in fp32.
 // `X` is x or dy; `Mt` is the group's B or C tile already transposed to [N][kQ] (tokens contiguous) by cb_kernel,
 // staged into LDS once per workgroup.  Per head only the x tile moves: it is loaded 16 bytes at a time, scaled in
 // fp32 and written transposed; the next head's tile is prefetched into registers while the MFMAs run.
-template <typename T, int P, int N, bool DSTATE>
+template <typename T, int P, int N, bool DSTATE, typename LT>
 __global__ void __launch_bounds__(256)
 chunk_state_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
-                   const T* __restrict__ Mt, float* __restrict__ out,
+                   const T* __restrict__ Mt, LT* __restrict__ out,
                    int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks, int64_t nslices, int64_t hps,
                    int64_t Xsb, int64_t Xsl, int64_t Xsh) {
     constexpr int LD = lds_ld<T>(kQ);
@@ -183,7 +186,7 @@ chunk_state_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
         floatx16 acc[BM][BN];
         acc_zero(acc);
         wave_mma<BM, BN>(acc, sX + wm * (P / 2) * LD, LD, sM + wn * (N / 2) * LD, LD, 0, kQ);
-        float* op = out + ((b * nchunks + c) * nheads + h) * (int64_t)(P * N);
+        LT* op = out + ((b * nchunks + c) * nheads + h) * (int64_t)(P * N);
 #pragma unroll
         for (int i = 0; i < BM; ++i)
 #pragma unroll
@@ -192,7 +195,7 @@ chunk_state_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
                 for (int v = 0; v < 16; ++v) {
                     const int row = wm * (P / 2) + i * 32 + acc_row(lane, v);
                     const int col = wn * (N / 2) + j * 32 + acc_col(lane);
-                    op[row * N + col] = acc[i][j][v];
+                    op[row * N + col] = from_f32<LT>(acc[i][j][v]);
                 }
     }
 }
@@ -216,9 +219,9 @@ chunk_state_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
 // the states), leaving an error that is constant over the chunk and accumulates in dA.
 constexpr int kScanSplit = 4;
 
-template <typename T, int PN, bool REVERSE>
+template <typename T, int PN, bool REVERSE, typename LT>
 __global__ void __launch_bounds__(256)
-state_scan_kernel(const float* __restrict__ local, const float* __restrict__ lam, const float* __restrict__ init,
+state_scan_kernel(const LT* __restrict__ local, const float* __restrict__ lam, const float* __restrict__ init,
                   T* __restrict__ prev, float* __restrict__ final_out,
                   const T* __restrict__ sprev, float* __restrict__ dlam,
                   int64_t nheads, int64_t nchunks) {
@@ -245,7 +248,8 @@ state_scan_kernel(const float* __restrict__ local, const float* __restrict__ lam
 #pragma unroll
         for (int e = 0; e < EPT; ++e) {
             const int off = part0 + (e * 256 + tid) * 4;
-            const floatx4 loc = *reinterpret_cast<const floatx4*>(local + tile + off);
+            float loc[4];
+            loadv<LT, 4>(local + tile + off, loc);
             // store the state entering (forward) / the gradient leaving (reverse) this chunk
             T o[4];
 #pragma unroll
