@@ -475,7 +475,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         auto dstates = [&](auto lt_tag) -> int {
             using LT = decltype(lt_tag);
             auto k = chunk_state_kernel<T, P, N, true, LT>;
-            const size_t sm = state_smem<T, P, N>();
+            const size_t sm = state_smem<T, P, N, LT>();
             int rc2;
             if ((rc2 = allow_smem(k, sm))) return rc2;
             int64_t ns, hps;

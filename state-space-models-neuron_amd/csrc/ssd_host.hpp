@@ -147,8 +147,8 @@ inline int allow_smem(K kernel, size_t bytes) {
     return M2_OK;
 }
 
-template <typename T, int P, int N>
-inline size_t state_smem() { return (size_t)(P + N) * lds_ld<T>(kQ) * sizeof(T); }
+template <typename T, int P, int N, typename LT>
+inline size_t state_smem() { return (size_t)(P + N) * lds_ld<T>(kQ) * sizeof(T) + (sizeof(LT) == 2 ? (size_t)4 * (P / 2) * (N / 2 + 8) * 2 : 0); }
 template <typename T>
 inline size_t cb_smem() { return (size_t)2 * kQ * lds_ld<T>(64) * sizeof(T); }
 
@@ -181,7 +181,7 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
     auto states = [&](auto lt_tag) -> int {
         using LT = decltype(lt_tag);
         auto k = chunk_state_kernel<T, P, N, false, LT>;
-        const size_t sm = state_smem<T, P, N>();
+        const size_t sm = state_smem<T, P, N, LT>();
         int rc2;
         if ((rc2 = allow_smem(k, sm))) return rc2;
         int64_t ns, hps;

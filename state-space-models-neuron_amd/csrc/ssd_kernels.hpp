@@ -144,6 +144,9 @@ chunk_state_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* sX = reinterpret_cast<T*>(smem_raw);        // [P][LD]   x^T scaled
     T* sM = sX + P * LD;                           // [N][LD]   B^T or C^T
+    constexpr bool PACK = sizeof(LT) == 2;         // 16-bit output: through a wave-private tile to 16-byte row stores
+    constexpr int LDO = N / 2 + 8;
+    LT* sO = reinterpret_cast<LT*>(sM + N * LD);   // PACK: [4 waves][P / 2][LDO]
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int64_t c = blockIdx.x, b = blockIdx.z;
     const int64_t g = blockIdx.y / nslices, slice = blockIdx.y % nslices;
@@ -187,16 +190,37 @@ chunk_state_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
         acc_zero(acc);
         wave_mma<BM, BN>(acc, sX + wm * (P / 2) * LD, LD, sM + wn * (N / 2) * LD, LD, 0, kQ);
         LT* op = out + ((b * nchunks + c) * nheads + h) * (int64_t)(P * N);
+        if (PACK) {
+            LT* sOw = sO + wave * (P / 2) * LDO;
 #pragma unroll
-        for (int i = 0; i < BM; ++i)
+            for (int i = 0; i < BM; ++i)
 #pragma unroll
-            for (int j = 0; j < BN; ++j)
+                for (int j = 0; j < BN; ++j)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int row = wm * (P / 2) + i * 32 + acc_row(lane, v);
-                    const int col = wn * (N / 2) + j * 32 + acc_col(lane);
-                    op[row * N + col] = from_f32<LT>(acc[i][j][v]);
-                }
+                    for (int v = 0; v < 16; ++v)
+                        sOw[(i * 32 + acc_row(lane, v)) * LDO + j * 32 + acc_col(lane)] = from_f32<LT>(acc[i][j][v]);
+            wave_lds_sync();
+            constexpr int LPR = (N / 2) / 8;           // lanes per row of this wave's [P/2][N/2] block (8 elements each)
+            constexpr int RPP = 64 / LPR;
+#pragma unroll
+            for (int ps = 0; ps < (P / 2) / RPP; ++ps) {
+                const int rl = ps * RPP + lane / LPR, cv = lane % LPR;
+                *reinterpret_cast<uint4*>(op + (wm * (P / 2) + rl) * N + wn * (N / 2) + cv * 8) =
+                    *reinterpret_cast<const uint4*>(sOw + rl * LDO + cv * 8);
+            }
+            wave_lds_sync();
+        } else {
+#pragma unroll
+            for (int i = 0; i < BM; ++i)
+#pragma unroll
+                for (int j = 0; j < BN; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int row = wm * (P / 2) + i * 32 + acc_row(lane, v);
+                        const int col = wn * (N / 2) + j * 32 + acc_col(lane);
+                        op[row * N + col] = from_f32<LT>(acc[i][j][v]);
+                    }
+        }
     }
 }
 
