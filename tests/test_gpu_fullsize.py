@@ -1,0 +1,101 @@
+"""GPU: size-independent properties at the full benchmark shapes (the fp64 oracle is too slow there).
+
+* sequence split: scanning the whole sequence == scanning its two halves with the final state of the first handed to
+  the second as initial state (forward), for the 2.7B (c1) and 7B-layer (c3) SSD shapes;
+* linearity of the backward in dy, and dD == sum(dy * x) (mamba2_kernel.py:471), at the c1 shape;
+* conv: shifting the input by one token shifts the output by one token (causality + time invariance), c2 shape;
+* decode: 4 token steps from the prefill's final state == the chunked scan over the 4 extra tokens, c4 width.
+"""
+import pytest
+import torch
+
+from conftest import rel_rms_err
+from oracle.ssd import make_ssd_inputs
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("b,l,h,p,n,g", [(4, 2048, 80, 64, 128, 1), (2, 4096, 128, 64, 128, 8)])
+def test_ssd_sequence_split_bf16(b, l, h, p, n, g):
+    from mamba2.mamba2_kernel import ssd_forward
+    d = make_ssd_inputs(b, l, h, p, n, g, seed=3, dtype=torch.bfloat16, device=DEV)
+    y, S = ssd_forward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], want_final_state=True)
+    m = l // 2 + 128 * 3 + 40          # not a chunk multiple
+    a = {k: d[k][:, :m] for k in ("dt", "X", "B", "C")}
+    z = {k: d[k][:, m:] for k in ("dt", "X", "B", "C")}
+    y1, S1 = ssd_forward(a["dt"], d["A"], a["X"], a["B"], a["C"], d["D"], want_final_state=True)
+    y2, S2 = ssd_forward(z["dt"], d["A"], z["X"], z["B"], z["C"], d["D"], initial_state=S1, want_final_state=True)
+    assert torch.isfinite(y.float()).all()
+    # both sides are bf16 computations, each within 2e-2 x RMS of the exact result (the parity bar): triangle inequality
+    assert rel_rms_err(torch.cat([y1, y2], dim=1), y.float()) < 4e-2
+    # the states are fp32 sums of MFMA products whose operands (dt * decay * x, B) were rounded to bf16, and the chunk
+    # boundaries of the two scans differ, so the rounded operands differ: same bound
+    assert rel_rms_err(S2, S) < 4e-2
+    assert (S2 - S).norm() / S.norm() < 5e-3
+
+
+def test_ssd_backward_linearity_c1():
+    from mamba2.mamba2_kernel import alloc_chunk_states, ssd_backward, ssd_forward
+    b, l, h, p, n, g = 4, 2048, 80, 64, 128, 1
+    d = make_ssd_inputs(b, l, h, p, n, g, seed=5, dtype=torch.bfloat16, device=DEV)
+    st = alloc_chunk_states(d["dt"], d["A"], d["X"], d["B"], d["C"])
+    ssd_forward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], chunk_states=st)
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    dy1 = torch.randn(b, l, h, p, device=DEV, generator=gen).to(torch.bfloat16)
+    dy2 = torch.randn(b, l, h, p, device=DEV, generator=gen).to(torch.bfloat16)
+    dys = (dy1.float() + dy2.float())
+    dy12 = dys.to(torch.bfloat16)
+    g1 = ssd_backward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], dy1, chunk_states=st)
+    g2 = ssd_backward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], dy2, chunk_states=st)
+    g12 = ssd_backward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], dy12, chunk_states=st)
+    for name, a_, b_, c_ in zip(("ddt", "dA", "dX", "dB", "dC", "dD"), g1, g2, g12):
+        assert torch.isfinite(c_.float()).all(), name
+        # three bf16 computations, each within 2e-2 x RMS of its exact gradient: triangle inequality on the maximum,
+        # and a tight bound on the relative L2 difference, which a wrong term or sign would break
+        assert rel_rms_err(c_.float(), a_.float() + b_.float()) < 6e-2, name
+        assert (c_.float() - a_.float() - b_.float()).norm() / c_.float().norm() < 1e-2, name
+    # dD_h = sum over batch, tokens and channels of dy * x  (mamba2_kernel.py:471)
+    dD_direct = (dy12.float() * d["X"].float()).sum(dim=(0, 1, 3))
+    assert rel_rms_err(g12[5], dD_direct) < 1e-3
+
+
+def test_conv_shift_equivariance_c2():
+    from mamba2.conv1d_grouped import conv1d_forward
+    from oracle.conv import make_conv_inputs
+    d = make_conv_inputs(4, 2048, 5376, 4, seed=2, dtype=torch.bfloat16, device=DEV)
+    y = conv1d_forward(d["x"], d["w"], d["bias"], "silu", channels_last=True)
+    xs = torch.zeros_like(d["x"])
+    xs[:, 1:] = d["x"][:, :-1]
+    ys = conv1d_forward(xs, d["w"], d["bias"], "silu", channels_last=True)
+    assert torch.equal(ys[:, 1:], y[:, :-1])
+    # a zero token in front sees only the bias
+    assert torch.equal(ys[:, 0], torch.nn.functional.silu(d["bias"].float()).to(torch.bfloat16).expand(4, -1))
+
+
+def test_decode_continues_prefill_c4_width():
+    # prefill l tokens with the chunked scan, then 4 decode steps == chunked scan over l + 4 tokens (last 4 outputs, final state)
+    from mamba2.mamba2_kernel import ssd_forward
+    from mamba2.mamba2_kernel_inference import mamba2_kernel_inference
+    b, l, h, p, n, g = 8, 256, 80, 64, 128, 1
+    extra = 4
+    d = make_ssd_inputs(b, l + extra, h, p, n, g, seed=7, dtype=torch.bfloat16, device=DEV)
+    y_all, S_all = ssd_forward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], want_final_state=True)
+    _, S = ssd_forward(d["dt"][:, :l], d["A"], d["X"][:, :l], d["B"][:, :l], d["C"][:, :l], d["D"], want_final_state=True)
+    # the decode step convolves and activates its input; an identity conv (weight 1 on the current token, no bias, no
+    # activation) hands x, B, C of the extra tokens to the state update unchanged
+    C = h * p + 2 * g * n
+    w = torch.zeros(C, 4, dtype=torch.bfloat16, device=DEV)
+    w[:, 3] = 1
+    conv_state = torch.zeros(b, C, 3, dtype=torch.bfloat16, device=DEV)
+    ys = []
+    for t in range(l, l + extra):
+        xBC = torch.cat([d["X"][:, t].reshape(b, -1), d["B"][:, t].reshape(b, -1), d["C"][:, t].reshape(b, -1)], dim=-1).unsqueeze(1)
+        y, conv_state, S = mamba2_kernel_inference(xBC.contiguous(), conv_state, w, None, S, d["dt"][:, t:t + 1].contiguous(), d["A"], d["D"],
+                                                   n_groups=g, activation=None)
+        ys.append(y)
+    y_dec = torch.cat(ys, dim=1).view(b, extra, h, p)
+    # the decode step works in fp32 on the bf16 inputs; the chunked scan rounds its MFMA operands to bf16
+    assert rel_rms_err(y_dec, y_all[:, l:].float()) < 2e-2
+    assert rel_rms_err(S, S_all) < 4e-2
+    assert (S - S_all).norm() / S_all.norm() < 5e-3
