@@ -64,6 +64,7 @@ template <int BYTES> struct RawBytes;
 template <> struct RawBytes<16> { using type = uint4; };
 template <> struct RawBytes<8> { using type = uint2; };
 template <> struct RawBytes<4> { using type = uint32_t; };
+template <> struct RawBytes<2> { using type = uint16_t; };
 template <typename T, int V> using RawVec = typename RawBytes<V * (int)sizeof(T)>::type;
 template <typename T, int V>
 __device__ __forceinline__ RawVec<T, V> loadv_raw(const T* __restrict__ p) { return *reinterpret_cast<const RawVec<T, V>*>(p); }
@@ -95,10 +96,12 @@ __device__ __forceinline__ void cvt16(const uint4& raw, float (&out)[VecTraits<T
     for (int i = 0; i < N; ++i) out[i] = to_f32(e[i]);
 }
 
-__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + __expf(-z)); }
+// sigmoid through the hardware reciprocal (1 ulp) rather than an IEEE division (ten more VALU instructions per element)
+__device__ __forceinline__ float sigmoid_f(float z) { return __builtin_amdgcn_rcpf(1.0f + __expf(-z)); }
+__device__ __forceinline__ float silu_f(float z) { return z * sigmoid_f(z); }
 // d/dz silu(z) = s * (1 + z * (1 - s)),  s = sigmoid(z)
 __device__ __forceinline__ float silu_grad_f(float z) {
-    float s = 1.0f / (1.0f + __expf(-z));
+    float s = sigmoid_f(z);
     return s * (1.0f + z * (1.0f - s));
 }
 

@@ -23,8 +23,11 @@ namespace m2 {
 namespace {
 
 constexpr int kMaxK = 8;
-#ifndef M2_CONV_TL
-#define M2_CONV_TL 64
+#ifndef M2_CONV_TLF
+#define M2_CONV_TLF 16
+#endif
+#ifndef M2_CONV_TLB
+#define M2_CONV_TLB 64
 #endif
 #ifndef M2_CONV_UNR
 #define M2_CONV_UNR 4
@@ -35,19 +38,23 @@ constexpr int kMaxK = 8;
 #ifndef M2_CONV_VB
 #define M2_CONV_VB 8
 #endif
-constexpr int kTL = M2_CONV_TL;      // tokens per thread in the fast path
+// Tokens per thread in the fast path.  The forward is short on loads in flight, so it takes short segments (many
+// threads); the backward carries more per-thread state and recomputes 3 lag tokens per segment, so it takes long ones.
+constexpr int kTLF = M2_CONV_TLF;
+constexpr int kTLB = M2_CONV_TLB;
 constexpr int kUNR = M2_CONV_UNR;    // tokens whose loads are in flight together
 #ifndef M2_CONV_CVT
-#define M2_CONV_CVT 32
+#define M2_CONV_CVT 64
 #endif
 #ifndef M2_CONV_SEG
-#define M2_CONV_SEG 8
+#define M2_CONV_SEG 4
 #endif
 #ifndef M2_CONV_NT
 #define M2_CONV_NT 1
 #endif
 constexpr int kCVT = M2_CONV_CVT;    // channel vectors per block (x dimension)
 constexpr int kSEG = M2_CONV_SEG;    // token segments per block (y dimension)
+static_assert(kTLF % kUNR == 0 && kTLB % kUNR == 0 && kUNR >= 3, "segments are whole load groups; the dx lag fits one group");
 
 // streaming loads/stores of the activations (optionally non-temporal: nothing is re-read soon enough to be worth caching)
 template <int BYTES> struct StreamVec;
@@ -80,28 +87,56 @@ __device__ __forceinline__ void st_param(void* p, int pd, int64_t i, float v) {
     else reinterpret_cast<bf16_t*>(p)[i] = from_f32<bf16_t>(v);
 }
 
+// The 4 taps and the bias of V consecutive channels with 16-byte loads, all in flight together (w is (C, 4) contiguous).
+template <typename WT, int V>
+__device__ __forceinline__ void load_taps(const void* __restrict__ w, const void* __restrict__ bias, int64_t c0,
+                                          float (&wv)[4][V], float (&bv)[V]) {
+    constexpr int TV = (V * 4 * (int)sizeof(WT)) < 16 ? V * 4 : 16 / (int)sizeof(WT);     // elements per tap load (<= 16 bytes)
+    constexpr int PER = 16 / (int)sizeof(WT);
+    static_assert((V * 4) % TV == 0, "taps of one thread must fill whole vectors");
+    const WT* wp = static_cast<const WT*>(w) + c0 * 4;
+    float flat[V * 4];
+#pragma unroll
+    for (int i = 0; i < V * 4 / TV; ++i) {
+        float tmp[TV];
+        loadv<WT, TV>(wp + i * TV, tmp);
+#pragma unroll
+        for (int e = 0; e < TV; ++e) flat[i * TV + e] = tmp[e];
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wv[i][j] = flat[j * 4 + i];
+        bv[j] = 0.f;
+    }
+    if (bias) {
+        constexpr int BV = V < PER ? V : PER;      // at most 16 bytes per load
+#pragma unroll
+        for (int i = 0; i < V / BV; ++i) {
+            float tmp[BV];
+            loadv<WT, BV>(static_cast<const WT*>(bias) + c0 + i * BV, tmp);
+#pragma unroll
+            for (int e = 0; e < BV; ++e) bv[i * BV + e] = tmp[e];
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // Fast path, channels-last, k == 4.
 // grid: x = ceil(CV / kCVT), y = ceil(nseg / kSEG), z = batch; block (kCVT, kSEG).
-template <typename T, int V, int ACT>
+template <typename T, typename WT, int V, int ACT>
 __global__ void __launch_bounds__(kCVT * kSEG)
 conv_fwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const void* __restrict__ bias,
-                   T* __restrict__ y, int64_t l, int64_t C, int64_t xsb, int64_t xsl, int64_t ysb, int64_t ysl,
-                   int pd) {
+                   T* __restrict__ y, int64_t l, int64_t C, int64_t xsb, int64_t xsl, int64_t ysb, int64_t ysl) {
     const int64_t cv = (int64_t)blockIdx.x * kCVT + threadIdx.x;
     const int64_t seg = (int64_t)blockIdx.y * kSEG + threadIdx.y;
     const int64_t b = blockIdx.z;
     const int64_t c0 = cv * V;
-    const int64_t t0 = seg * kTL;
+    const int64_t t0 = seg * kTLF;
     if (c0 >= C || t0 >= l) return;
 
     float wv[4][V], bv[V];
-#pragma unroll
-    for (int j = 0; j < V; ++j) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) wv[i][j] = ld_param(w, pd, (c0 + j) * 4 + i);
-        bv[j] = bias ? ld_param(bias, pd, c0 + j) : 0.f;
-    }
+    load_taps<WT, V>(w, bias, c0, wv, bv);
     const T* xp = x + b * xsb + c0;
     T* yp = y + b * ysb + c0;
     float h0[V], h1[V], h2[V];   // x[t-3], x[t-2], x[t-1]
@@ -110,9 +145,40 @@ conv_fwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const vo
     if (t0 - 3 >= 0) loadv<T, V>(xp + (t0 - 3) * xsl, h0);
     if (t0 - 2 >= 0) loadv<T, V>(xp + (t0 - 2) * xsl, h1);
     if (t0 - 1 >= 0) loadv<T, V>(xp + (t0 - 1) * xsl, h2);
-    const int64_t t1 = (t0 + kTL < l) ? t0 + kTL : l;
+    auto step = [&](const RawVec<T, V>& r, T* __restrict__ yq) {
+        float out[V], cur[V];
+        cvtv<T, V>(r, cur);
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            float z = bv[j] + wv[0][j] * h0[j] + wv[1][j] * h1[j] + wv[2][j] * h2[j] + wv[3][j] * cur[j];
+            out[j] = act_f<ACT>(z);
+            h0[j] = h1[j]; h1[j] = h2[j]; h2[j] = cur[j];
+        }
+        st_stream<T, V>(yq, out);
+    };
     // software pipeline: the loads of group g+1 are issued before group g is computed and stored
     RawVec<T, V> nxt[kUNR];
+    if (t0 + kTLF <= l) {
+        // whole segment inside the sequence: no per-token predicates, so the wait before a group's compute can leave
+        // the previous group's stores in flight
+        const T* xq = xp + t0 * xsl;
+        T* yq = yp + t0 * ysl;
+#pragma unroll
+        for (int u = 0; u < kUNR; ++u) nxt[u] = ld_stream<T, V>(xq + u * xsl);
+        for (int g = 0; g < kTLF / kUNR - 1; ++g) {
+            RawVec<T, V> raw[kUNR];
+            xq += kUNR * xsl;
+#pragma unroll
+            for (int u = 0; u < kUNR; ++u) { raw[u] = nxt[u]; nxt[u] = ld_stream<T, V>(xq + u * xsl); }
+#pragma unroll
+            for (int u = 0; u < kUNR; ++u) step(raw[u], yq + u * ysl);
+            yq += kUNR * ysl;
+        }
+#pragma unroll
+        for (int u = 0; u < kUNR; ++u) step(nxt[u], yq + u * ysl);
+        return;
+    }
+    const int64_t t1 = l;
 #pragma unroll
     for (int u = 0; u < kUNR; ++u)
         if (t0 + u < t1) nxt[u] = ld_stream<T, V>(xp + (t0 + u) * xsl);
@@ -124,37 +190,26 @@ conv_fwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const vo
         for (int u = 0; u < kUNR; ++u)
             if (tg + kUNR + u < t1) nxt[u] = ld_stream<T, V>(xp + (tg + kUNR + u) * xsl);
 #pragma unroll
-        for (int u = 0; u < kUNR; ++u) {
-            if (tg + u < t1) {
-                float out[V], cur[V];
-                cvtv<T, V>(raw[u], cur);
-#pragma unroll
-                for (int j = 0; j < V; ++j) {
-                    float z = bv[j] + wv[0][j] * h0[j] + wv[1][j] * h1[j] + wv[2][j] * h2[j] + wv[3][j] * cur[j];
-                    out[j] = act_f<ACT>(z);
-                    h0[j] = h1[j]; h1[j] = h2[j]; h2[j] = cur[j];
-                }
-                st_stream<T, V>(yp + (tg + u) * ysl, out);
-            }
-        }
+        for (int u = 0; u < kUNR; ++u)
+            if (tg + u < t1) step(raw[u], yp + (tg + u) * ysl);
     }
 }
 
 // Backward fast path.  Each thread marches t over [t0, t0+TL+3): at step t it forms g[t] and
 // emits dx[t-3] = w3 g[t-3] + w2 g[t-2] + w1 g[t-1] + w0 g[t]  (dx[s] = sum_i w[i] g[s+3-i]).
 // Partials: part[(blockIdx.z * gridDim.y + blockIdx.y)][c][0..4] = (dw0..dw3, db).
-template <typename T, int V, int ACT>
+template <typename T, typename WT, int V, int ACT>
 __global__ void __launch_bounds__(kCVT * kSEG)
 conv_bwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const void* __restrict__ bias,
                    const T* __restrict__ dy, T* __restrict__ dx, float* __restrict__ part,
                    int64_t l, int64_t C, int64_t xsb, int64_t xsl, int64_t gsb, int64_t gsl,
-                   int64_t dsb, int64_t dsl, int pd) {
+                   int64_t dsb, int64_t dsl) {
     __shared__ float red[kSEG][5][kCVT * V + 1];
     const int64_t cv = (int64_t)blockIdx.x * kCVT + threadIdx.x;
     const int64_t seg = (int64_t)blockIdx.y * kSEG + threadIdx.y;
     const int64_t b = blockIdx.z;
     const int64_t c0 = cv * V;
-    const int64_t t0 = seg * kTL;
+    const int64_t t0 = seg * kTLB;
     const bool active = (c0 < C) && (t0 < l);
 
     float acc[5][V];
@@ -165,12 +220,7 @@ conv_bwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const vo
 
     if (active) {
         float wv[4][V], bv[V];
-#pragma unroll
-        for (int j = 0; j < V; ++j) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) wv[i][j] = ld_param(w, pd, (c0 + j) * 4 + i);
-            bv[j] = bias ? ld_param(bias, pd, c0 + j) : 0.f;
-        }
+        load_taps<WT, V>(w, bias, c0, wv, bv);
         const T* xp = x + b * xsb + c0;
         const T* gp = dy + b * gsb + c0;
         T* dp = dx + b * dsb + c0;
@@ -181,58 +231,83 @@ conv_bwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const vo
         if (t0 - 3 >= 0) loadv<T, V>(xp + (t0 - 3) * xsl, h0);
         if (t0 - 2 >= 0) loadv<T, V>(xp + (t0 - 2) * xsl, h1);
         if (t0 - 1 >= 0) loadv<T, V>(xp + (t0 - 1) * xsl, h2);
-        const int64_t tseg = (t0 + kTL < l) ? t0 + kTL : l;      // end of this thread's own tokens
-        const int64_t tend = tseg + 3;                            // march 3 further for the dx lag
+        // one token: g[t] from x[t-3..t] and dy[t]; the weight/bias sums if the token is this thread's own; dx[t-3] to dq if emit
+        auto step = [&](const RawVec<T, V>& rx, const RawVec<T, V>& rg, bool own, bool emit, T* __restrict__ dq) {
+            float g[V], cur[V], gy[V];
+            cvtv<T, V>(rx, cur);
+            cvtv<T, V>(rg, gy);
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                float z = bv[j] + wv[0][j] * h0[j] + wv[1][j] * h1[j] + wv[2][j] * h2[j] + wv[3][j] * cur[j];
+                g[j] = gy[j] * act_grad_f<ACT>(z);     // gy == 0 beyond the sequence end
+                if (own) {
+                    acc[0][j] += h0[j] * g[j];
+                    acc[1][j] += h1[j] * g[j];
+                    acc[2][j] += h2[j] * g[j];
+                    acc[3][j] += cur[j] * g[j];
+                    acc[4][j] += g[j];
+                }
+            }
+            if (emit) {
+                float o[V];
+#pragma unroll
+                for (int j = 0; j < V; ++j)
+                    o[j] = wv[3][j] * g0[j] + wv[2][j] * g1[j] + wv[1][j] * g2[j] + wv[0][j] * g[j];
+                st_stream<T, V>(dq, o);
+            }
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                h0[j] = h1[j]; h1[j] = h2[j]; h2[j] = cur[j];
+                g0[j] = g1[j]; g1[j] = g2[j]; g2[j] = g[j];
+            }
+        };
         // software pipeline: the loads of group g+1 are issued before group g is computed and stored
         RawVec<T, V> nx[kUNR], ng[kUNR];
+        if (t0 + kTLB + kUNR <= l) {
+            // the segment and its 3 lag tokens lie inside the sequence: no per-token predicates
+            const T* xq = xp + t0 * xsl;
+            const T* gq = gp + t0 * gsl;
+            T* dq = dp + (t0 - 3) * dsl;
 #pragma unroll
-        for (int u = 0; u < kUNR; ++u) {
-            const int64_t t = t0 + u;
-            if (t < tend && t < l) { nx[u] = ld_stream<T, V>(xp + t * xsl); ng[u] = ld_stream<T, V>(gp + t * gsl); }
-            else { nx[u] = RawVec<T, V>{}; ng[u] = RawVec<T, V>{}; }
-        }
-        for (int64_t tg = t0; tg < tend; tg += kUNR) {
-            RawVec<T, V> rawx[kUNR], rawg[kUNR];
+            for (int u = 0; u < kUNR; ++u) { nx[u] = ld_stream<T, V>(xq + u * xsl); ng[u] = ld_stream<T, V>(gq + u * gsl); }
+            for (int grp = 0; grp < kTLB / kUNR; ++grp) {
+                RawVec<T, V> rawx[kUNR], rawg[kUNR];
+                xq += kUNR * xsl;
+                gq += kUNR * gsl;
 #pragma unroll
-            for (int u = 0; u < kUNR; ++u) { rawx[u] = nx[u]; rawg[u] = ng[u]; }
+                for (int u = 0; u < kUNR; ++u) {
+                    rawx[u] = nx[u]; rawg[u] = ng[u];
+                    nx[u] = ld_stream<T, V>(xq + u * xsl); ng[u] = ld_stream<T, V>(gq + u * gsl);
+                }
+#pragma unroll
+                for (int u = 0; u < kUNR; ++u) step(rawx[u], rawg[u], true, grp > 0 || u >= 3, dq + u * dsl);
+                dq += kUNR * dsl;
+            }
+#pragma unroll
+            for (int u = 0; u < 3; ++u) step(nx[u], ng[u], false, true, dq + u * dsl);
+        } else {
+            const int64_t tseg = (t0 + kTLB < l) ? t0 + kTLB : l;      // end of this thread's own tokens
+            const int64_t tend = tseg + 3;                            // march 3 further for the dx lag
 #pragma unroll
             for (int u = 0; u < kUNR; ++u) {
-                const int64_t t = tg + kUNR + u;
+                const int64_t t = t0 + u;
                 if (t < tend && t < l) { nx[u] = ld_stream<T, V>(xp + t * xsl); ng[u] = ld_stream<T, V>(gp + t * gsl); }
                 else { nx[u] = RawVec<T, V>{}; ng[u] = RawVec<T, V>{}; }
             }
+            for (int64_t tg = t0; tg < tend; tg += kUNR) {
+                RawVec<T, V> rawx[kUNR], rawg[kUNR];
 #pragma unroll
-            for (int u = 0; u < kUNR; ++u) {
-                const int64_t t = tg + u;
-                if (t < tend) {
-                    const bool own = t < tseg;
-                    float g[V], cur[V], gy[V];
-                    cvtv<T, V>(rawx[u], cur);
-                    cvtv<T, V>(rawg[u], gy);
+                for (int u = 0; u < kUNR; ++u) { rawx[u] = nx[u]; rawg[u] = ng[u]; }
 #pragma unroll
-                    for (int j = 0; j < V; ++j) {
-                        float z = bv[j] + wv[0][j] * h0[j] + wv[1][j] * h1[j] + wv[2][j] * h2[j] + wv[3][j] * cur[j];
-                        g[j] = gy[j] * act_grad_f<ACT>(z);     // gy == 0 beyond the sequence end
-                        if (own) {
-                            acc[0][j] += h0[j] * g[j];
-                            acc[1][j] += h1[j] * g[j];
-                            acc[2][j] += h2[j] * g[j];
-                            acc[3][j] += cur[j] * g[j];
-                            acc[4][j] += g[j];
-                        }
-                    }
-                    if (t - 3 >= t0) {
-                        float o[V];
+                for (int u = 0; u < kUNR; ++u) {
+                    const int64_t t = tg + kUNR + u;
+                    if (t < tend && t < l) { nx[u] = ld_stream<T, V>(xp + t * xsl); ng[u] = ld_stream<T, V>(gp + t * gsl); }
+                    else { nx[u] = RawVec<T, V>{}; ng[u] = RawVec<T, V>{}; }
+                }
 #pragma unroll
-                        for (int j = 0; j < V; ++j)
-                            o[j] = wv[3][j] * g0[j] + wv[2][j] * g1[j] + wv[1][j] * g2[j] + wv[0][j] * g[j];
-                        st_stream<T, V>(dp + (t - 3) * dsl, o);
-                    }
-#pragma unroll
-                    for (int j = 0; j < V; ++j) {
-                        h0[j] = h1[j]; h1[j] = h2[j]; h2[j] = cur[j];
-                        g0[j] = g1[j]; g1[j] = g2[j]; g2[j] = g[j];
-                    }
+                for (int u = 0; u < kUNR; ++u) {
+                    const int64_t t = tg + u;
+                    if (t < tend) step(rawx[u], rawg[u], t < tseg, t - 3 >= t0, dp + (t - 3) * dsl);
                 }
             }
         }
@@ -255,6 +330,12 @@ conv_bwd_cl_kernel(const T* __restrict__ x, const void* __restrict__ w, const vo
             part[(pslot * C + c) * 5 + i] = s;
         }
     }
+}
+
+// Zero fill (a kernel rather than a memset node, so that a caller may capture the call in a graph).
+__global__ void conv_zero_kernel(uint16_t* __restrict__ p, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
 }
 
 // Second stage: sum the per-block partials.  One thread per (channel, tap-or-bias).
@@ -374,6 +455,7 @@ bool fast_path_ok(const m2_conv1d_params* p, bool bwd) {
     if (p->x_stride_b % V || p->x_stride_l % V || p->y_stride_b % V || p->y_stride_l % V) return false;
     auto al = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) % (V * sizeof(T))) == 0; };
     if (!al(p->x)) return false;
+    if (reinterpret_cast<uintptr_t>(p->w) % 16 || reinterpret_cast<uintptr_t>(p->bias) % 16) return false;   // vector tap loads
     if (!bwd && !al(p->y)) return false;
     if (bwd) {
         if (p->dx_stride_c != 1 || p->dx_stride_b % V || p->dx_stride_l % V) return false;
@@ -400,15 +482,18 @@ int launch_fwd(const m2_conv1d_params* p, hipStream_t st) {
     T* y = static_cast<T*>(p->y);
     constexpr int V = conv_vec<T>(false);
     if (fast_path_ok<T, V>(p, false) && p->activation != M2_ACT_RELU) {
-        const int64_t CV = C / V, nseg = ceil_div(l, kTL);
+        const int64_t CV = C / V, nseg = ceil_div(l, kTLF);
         dim3 grid((unsigned)ceil_div(CV, kCVT), (unsigned)ceil_div(nseg, kSEG), (unsigned)nb), block(kCVT, kSEG);
         M2_REQUIRE(grid.y <= 65535, M2_ERR_SHAPE, "conv1d: sequence too long for the grid");
-        if (p->activation == M2_ACT_SILU)
-            conv_fwd_cl_kernel<T, V, M2_ACT_SILU><<<grid, block, 0, st>>>(x, p->w, p->bias, y, l, C, p->x_stride_b, p->x_stride_l,
-                                                                        p->y_stride_b, p->y_stride_l, p->param_dtype);
-        else
-            conv_fwd_cl_kernel<T, V, M2_ACT_NONE><<<grid, block, 0, st>>>(x, p->w, p->bias, y, l, C, p->x_stride_b, p->x_stride_l,
-                                                                        p->y_stride_b, p->y_stride_l, p->param_dtype);
+        auto go = [&](auto kern) {
+            kern<<<grid, block, 0, st>>>(x, p->w, p->bias, y, l, C, p->x_stride_b, p->x_stride_l, p->y_stride_b, p->y_stride_l);
+        };
+        const bool silu = p->activation == M2_ACT_SILU;
+        if (p->param_dtype == M2_F32) {
+            if (silu) go(conv_fwd_cl_kernel<T, float, V, M2_ACT_SILU>); else go(conv_fwd_cl_kernel<T, float, V, M2_ACT_NONE>);
+        } else {
+            if (silu) go(conv_fwd_cl_kernel<T, bf16_t, V, M2_ACT_SILU>); else go(conv_fwd_cl_kernel<T, bf16_t, V, M2_ACT_NONE>);
+        }
     } else {
         const int64_t total = nb * l * C;
         const int tf = (p->x_stride_l == 1 && p->x_stride_c != 1) ? 1 : 0;
@@ -427,7 +512,7 @@ int launch_bwd(const m2_conv1d_params* p, hipStream_t st) {
     T* dx = static_cast<T*>(p->dx);
     constexpr int V = conv_vec<T>(true);
     if (fast_path_ok<T, V>(p, true) && p->activation != M2_ACT_RELU) {
-        const int64_t CV = C / V, nseg = ceil_div(l, kTL);
+        const int64_t CV = C / V, nseg = ceil_div(l, kTLB);
         dim3 grid((unsigned)ceil_div(CV, kCVT), (unsigned)ceil_div(nseg, kSEG), (unsigned)nb), block(kCVT, kSEG);
         M2_REQUIRE(grid.y <= 65535, M2_ERR_SHAPE, "conv1d: sequence too long for the grid");
         const int64_t nslots = (int64_t)grid.y * grid.z;
@@ -435,12 +520,16 @@ int launch_bwd(const m2_conv1d_params* p, hipStream_t st) {
         M2_REQUIRE(p->workspace && p->workspace_bytes >= need, M2_ERR_WORKSPACE,
                    "conv1d_bwd: workspace %zu bytes < %zu needed", p->workspace_bytes, need);
         float* part = static_cast<float*>(p->workspace);
-        if (p->activation == M2_ACT_SILU)
-            conv_bwd_cl_kernel<T, V, M2_ACT_SILU><<<grid, block, 0, st>>>(x, p->w, p->bias, dy, dx, part, l, C, p->x_stride_b, p->x_stride_l,
-                                                                        p->y_stride_b, p->y_stride_l, p->dx_stride_b, p->dx_stride_l, p->param_dtype);
-        else
-            conv_bwd_cl_kernel<T, V, M2_ACT_NONE><<<grid, block, 0, st>>>(x, p->w, p->bias, dy, dx, part, l, C, p->x_stride_b, p->x_stride_l,
-                                                                        p->y_stride_b, p->y_stride_l, p->dx_stride_b, p->dx_stride_l, p->param_dtype);
+        auto go = [&](auto kern) {
+            kern<<<grid, block, 0, st>>>(x, p->w, p->bias, dy, dx, part, l, C, p->x_stride_b, p->x_stride_l, p->y_stride_b, p->y_stride_l,
+                                         p->dx_stride_b, p->dx_stride_l);
+        };
+        const bool silu = p->activation == M2_ACT_SILU;
+        if (p->param_dtype == M2_F32) {
+            if (silu) go(conv_bwd_cl_kernel<T, float, V, M2_ACT_SILU>); else go(conv_bwd_cl_kernel<T, float, V, M2_ACT_NONE>);
+        } else {
+            if (silu) go(conv_bwd_cl_kernel<T, bf16_t, V, M2_ACT_SILU>); else go(conv_bwd_cl_kernel<T, bf16_t, V, M2_ACT_NONE>);
+        }
         int rc = check_launch("conv1d_bwd");
         if (rc) return rc;
         conv_reduce_partials_kernel<<<(unsigned)ceil_div(C * 5, 256), 256, 0, st>>>(part, nslots, C, 4, p->dw, p->db, p->param_dtype);
@@ -476,7 +565,7 @@ extern "C" int m2_conv1d_fwd(const m2_conv1d_params* p, void* stream) {
 extern "C" size_t m2_conv1d_bwd_workspace_bytes(int64_t batch, int64_t seqlen, int64_t channels, int32_t k) {
     using namespace m2;
     (void)k;
-    const int64_t nseg = ceil_div(seqlen, kTL);
+    const int64_t nseg = ceil_div(seqlen, kTLB);
     return (size_t)(ceil_div(nseg, kSEG) * batch * channels * 5) * sizeof(float) + 16;
 }
 
@@ -490,9 +579,10 @@ extern "C" int m2_conv1d_bwd(const m2_conv1d_params* p, void* stream) {
         // empty reduction: gradients of the parameters are zero
         hipStream_t st = static_cast<hipStream_t>(stream);
         const size_t esz = p->param_dtype == M2_F32 ? 4 : 2;
-        if (hipMemsetAsync(p->dw, 0, (size_t)p->channels * p->k * esz, st) != hipSuccess) return fail(M2_ERR_LAUNCH, "memset dw");
-        if (p->db && hipMemsetAsync(p->db, 0, (size_t)p->channels * esz, st) != hipSuccess) return fail(M2_ERR_LAUNCH, "memset db");
-        return M2_OK;
+        const int64_t nw = p->channels * p->k * (int64_t)(esz / 2), nb = p->channels * (int64_t)(esz / 2);     // 16-bit words
+        conv_zero_kernel<<<(unsigned)ceil_div(nw, (int64_t)256), 256, 0, st>>>(static_cast<uint16_t*>(p->dw), nw);
+        if (p->db) conv_zero_kernel<<<(unsigned)ceil_div(nb, (int64_t)256), 256, 0, st>>>(static_cast<uint16_t*>(p->db), nb);
+        return check_launch("conv1d_bwd_zero");
     }
     M2_REQUIRE(p->x && p->w && p->dy && p->dx, M2_ERR_NULL, "conv1d_bwd: x, w, dy, dx are required");
     M2_DISPATCH_DTYPE(p->dtype, T, return launch_bwd<T>(p, static_cast<hipStream_t>(stream)));
