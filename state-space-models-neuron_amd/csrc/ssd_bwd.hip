@@ -499,7 +499,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
             auto k = dg16_kernel<T, P>;
             const size_t sm = dg16_smem<P>();
             if ((rc = allow_smem(k, sm))) return rc;
-            k<<<grid_g, 512, sm, st>>>(x, w.ldtab, dy, w.G, w.dGp, w.dl,
+            k<<<grid_g, kDgWaves * 64, sm, st>>>(x, w.ldtab, dy, w.G, w.dGp, w.dl,
                                        p->seqlen, p->nheads, p->ngroups, nc, w.ns_g, w.hps_g,
                                        p->x_stride_b, p->x_stride_l, p->x_stride_h,
                                        p->dy_stride_b, p->dy_stride_l, p->dy_stride_h);

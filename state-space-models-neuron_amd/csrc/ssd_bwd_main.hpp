@@ -97,7 +97,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
 #pragma unroll
         for (int it = 0; it < NS; ++it) {
             const int s = (int)(wave_u * NS + it) * 64 + ln;
-            const int row = s / SPR_S, cs = (s % SPR_S) ^ swz_s<SPR_S>(row);
+            const int row = s / SPR_S, cs = (s % SPR_S) ^ tile_swz<SPR_S>(row);
             const uint32_t off = (uint32_t)(row * N + cs * 8) * 2u;
             async_copy16(Sp, off, dst + (wave_u * NS + it) * 1024u);
             async_copy16(Pp, off, dst + (uint32_t)(P * N * 2) + (wave_u * NS + it) * 1024u);
@@ -107,7 +107,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
 #pragma unroll
         for (int it = 0; it < NX; ++it) {
             const int s = (int)(wave_u * NX + it) * 64 + ln;
-            const int row = s / SPR_X, cs = (s % SPR_X) ^ swz_x(row);
+            const int row = s / SPR_X, cs = (s % SPR_X) ^ tile_swz<SPR_X>(row);
             const int grow = row < valid ? row : valid - 1;       // rows past the end: finite stand-ins, masked by zero scales
             async_copy16(Yp, (uint32_t)(grow * a.dy_sl + cs * 8) * 2u, dst + (uint32_t)(2 * P * N * 2) + (wave_u * NX + it) * 1024u);
             async_copy16(Xp, (uint32_t)(grow * a.x_sl + cs * 8) * 2u, dst + (uint32_t)((2 * P * N + kQ * P) * 2) + (wave_u * NX + it) * 1024u);
@@ -179,7 +179,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                     for (int j = 0; j < BN; ++j) {
                         const int col = j * 32 + tr_col;
                         const tvec4 zv = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-                            (M2_LDS tvec4*)(Z + (tok * SPR_X + ((col >> 3) ^ swz_x(tok))) * 8 + (col & 7)));
+                            (M2_LDS tvec4*)(Z + (tok * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(tok))) * 8 + (col & 7)));
 #pragma unroll
                         for (int e = 0; e < 4; ++e) s4[e] += t[0][j][4 * q + e] * to_f32(zv[e]);
                     }
@@ -197,7 +197,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
 #pragma unroll
                     for (int j = 0; j < BN; ++j) {
                         const int row = j * 32 + r;
-                        const Frag<T> bf = load_frag(cP + (row * SPR_S + ((ks * 2 + half) ^ swz_s<SPR_S>(row))) * 8);
+                        const Frag<T> bf = load_frag(cP + (row * SPR_S + ((ks * 2 + half) ^ tile_swz<SPR_S>(row))) * 8);
                         mma_frag(yo[0][j], ks < KCR ? foC[ks < KCR ? ks : 0] : load_frag(sFCw + r * LDC + (ks - KCR) * 16 + half * 8), bf);
                     }
                 }
@@ -222,7 +222,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
 #pragma unroll
                 for (int j = 0; j < BN; ++j) {
                     const int row = j * 32 + r;
-                    const Frag<T> bf = load_frag(cS + (row * SPR_S + ((ks * 2 + half) ^ swz_s<SPR_S>(row))) * 8);
+                    const Frag<T> bf = load_frag(cS + (row * SPR_S + ((ks * 2 + half) ^ tile_swz<SPR_S>(row))) * 8);
                     mma_frag(acc[0][j], foB[ks], bf);
                 }
             }
@@ -273,9 +273,9 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                     const int col = j * 32 + tr_col;
                     const int ta = ks * 16 + 8 * half + tr_row, tb = ta + 4;
                     const tvec4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-                        (M2_LDS tvec4*)(cY + (ta * SPR_X + ((col >> 3) ^ swz_x(ta))) * 8 + (col & 7)));
+                        (M2_LDS tvec4*)(cY + (ta * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(ta))) * 8 + (col & 7)));
                     const tvec4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-                        (M2_LDS tvec4*)(cY + (tb * SPR_X + ((col >> 3) ^ swz_x(tb))) * 8 + (col & 7)));
+                        (M2_LDS tvec4*)(cY + (tb * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(tb))) * 8 + (col & 7)));
                     Frag<T> bf;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) { bf.v[e] = lo[e]; bf.v[4 + e] = hi[e]; }
@@ -303,7 +303,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                     const int tok = row0 + 8 * q + rl;
                     const floatx4 ya = *reinterpret_cast<const floatx4*>(sYw + rl * P + cv * 8);
                     const floatx4 yb = *reinterpret_cast<const floatx4*>(sYw + rl * P + cv * 8 + 4);
-                    const int slot = cv ^ swz_x(tok);
+                    const int slot = cv ^ tile_swz<SPR_X>(tok);
                     const uint4 xr = *reinterpret_cast<const uint4*>(cX + (tok * SPR_X + slot) * 8);
                     const uint4 gr = *reinterpret_cast<const uint4*>(cY + (tok * SPR_X + slot) * 8);
                     const T* xe = reinterpret_cast<const T*>(&xr);
@@ -372,13 +372,13 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                     for (int ks = 0; ks < KSP; ++ks) {
                         const int pa = ks * 16 + 8 * half + tr_row, pb = pa + 4;
                         const tvec4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-                            (M2_LDS tvec4*)(St + (pa * SPR_S + ((col >> 3) ^ swz_s<SPR_S>(pa))) * 8 + (col & 7)));
+                            (M2_LDS tvec4*)(St + (pa * SPR_S + ((col >> 3) ^ tile_swz<SPR_S>(pa))) * 8 + (col & 7)));
                         const tvec4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-                            (M2_LDS tvec4*)(St + (pb * SPR_S + ((col >> 3) ^ swz_s<SPR_S>(pb))) * 8 + (col & 7)));
+                            (M2_LDS tvec4*)(St + (pb * SPR_S + ((col >> 3) ^ tile_swz<SPR_S>(pb))) * 8 + (col & 7)));
                         Frag<T> bf;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) { bf.v[e] = lo[e]; bf.v[4 + e] = hi[e]; }
-                        mma_frag(t, load_frag(Rows + (tok * SPR_X + ((ks * 2 + half) ^ swz_x(tok))) * 8), bf);
+                        mma_frag(t, load_frag(Rows + (tok * SPR_X + ((ks * 2 + half) ^ tile_swz<SPR_X>(tok))) * 8), bf);
                     }
 #pragma unroll
                     for (int v = 0; v < 16; ++v) accum[0][jn][v] += t[v] * ws[v];

@@ -70,9 +70,19 @@ __device__ __forceinline__ void async_copy_ldtab(const float* __restrict__ ldtab
     async_copy16(ldtab + bhc * (2 * kQ), (threadIdx.x & 63) * 16u, lds_addr);
 }
 
-// 16-byte slot s of row `row` lives at slot (s ^ swz) of that row
-template <int SPR> __device__ __forceinline__ int swz_s(int row) { return row & (SPR - 1); }          // S_prev tile
-__device__ __forceinline__ int swz_x(int row) { return ((row >> 1) & 1) << 2; }                      // x tile
+// 16-byte slot s of row `row` lives at slot (s ^ tile_swz(row)) of that row: the XOR applied to the slot index
+// inside a tile row of SPR slots.  The LDS serves 64 banks x 4 bytes per clock,
+// i.e. 16 lanes of a 16-byte read or 32 lanes of an 8-byte transpose read, and both access patterns of these tiles
+// must spread over all banks:
+//   row-wise fragments : 16 consecutive rows, one slot each          -> 16 different (row parity, slot) bank groups
+//   transpose reads    : 4 consecutive rows (aligned), 4 slots each   -> the rows' 4-slot groups must differ
+// which a bit permutation of the row index gives (256-byte rows: swap the two low bit pairs; 128-byte rows: bit 0
+// already selects the bank half, bits 1..3 go to slot bits 2, 0, 1).
+template <int SPR> __device__ __forceinline__ int tile_swz(int row) {
+    static_assert(SPR == 8 || SPR == 16, "tile rows of 128 or 256 bytes");
+    if (SPR == 16) return ((row & 3) << 2) | ((row >> 2) & 3);
+    return (((row >> 1) & 1) << 2) | (((row >> 3) & 1) << 1) | ((row >> 2) & 1);
+}
 
 template <int P, int N>
 constexpr size_t y16_smem() {
@@ -112,13 +122,13 @@ ssd_y16_kernel(const DiagArgs a) {
 #pragma unroll
     for (int it = 0; it < NS; ++it) {
         const int s = (wave * NS + it) * 64 + lane;
-        const int row = s / SPR_S, cs = (s % SPR_S) ^ swz_s<SPR_S>(row);
+        const int row = s / SPR_S, cs = (s % SPR_S) ^ tile_swz<SPR_S>(row);
         offS[it] = (uint32_t)(row * N + cs * 8) * 2u;
     }
 #pragma unroll
     for (int it = 0; it < NX; ++it) {
         const int s = (wave * NX + it) * 64 + lane;
-        const int row = s / SPR_X, cs = (s % SPR_X) ^ swz_x(row);
+        const int row = s / SPR_X, cs = (s % SPR_X) ^ tile_swz<SPR_X>(row);
         // rows past the end of the sequence re-read the last valid row: their dt is 0, so they only ever meet zeros
         const int grow = row < valid ? row : valid - 1;
         offX[it] = (uint32_t)(grow * a.Z_sl + cs * 8) * 2u;
@@ -187,7 +197,7 @@ ssd_y16_kernel(const DiagArgs a) {
 #pragma unroll
             for (int j = 0; j < BN; ++j) {
                 const int row = j * 32 + r;
-                const Frag<T> bf = load_frag(cS + (row * SPR_S + ((ks * 2 + half) ^ swz_s<SPR_S>(row))) * 8);
+                const Frag<T> bf = load_frag(cS + (row * SPR_S + ((ks * 2 + half) ^ tile_swz<SPR_S>(row))) * 8);
                 mma_frag(acc[0][j], fo[ks], bf);
             }
         }
@@ -229,9 +239,9 @@ ssd_y16_kernel(const DiagArgs a) {
                 const int ta = ks * 16 + tr_tok, tb = ta + 4;
                 typedef T tvec4 __attribute__((ext_vector_type(4)));
                 const tvec4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-                    (M2_LDS tvec4*)(cX + (ta * SPR_X + ((col >> 3) ^ swz_x(ta))) * 8 + (col & 7)));
+                    (M2_LDS tvec4*)(cX + (ta * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(ta))) * 8 + (col & 7)));
                 const tvec4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-                    (M2_LDS tvec4*)(cX + (tb * SPR_X + ((col >> 3) ^ swz_x(tb))) * 8 + (col & 7)));
+                    (M2_LDS tvec4*)(cX + (tb * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(tb))) * 8 + (col & 7)));
                 Frag<T> bf;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) { bf.v[e] = lo[e]; bf.v[4 + e] = hi[e]; }
@@ -257,7 +267,7 @@ ssd_y16_kernel(const DiagArgs a) {
                 const int tok = row0 + 8 * q + rl;
                 const floatx4 ya = *reinterpret_cast<const floatx4*>(sYw + rl * P + cv * 8);
                 const floatx4 yb = *reinterpret_cast<const floatx4*>(sYw + rl * P + cv * 8 + 4);
-                const uint4 xr = *reinterpret_cast<const uint4*>(cX + (tok * SPR_X + (cv ^ swz_x(tok))) * 8);
+                const uint4 xr = *reinterpret_cast<const uint4*>(cX + (tok * SPR_X + (cv ^ tile_swz<SPR_X>(tok))) * 8);
                 const T* xe = reinterpret_cast<const T*>(&xr);
                 uint4 o;
                 T* oe = reinterpret_cast<T*>(&o);
