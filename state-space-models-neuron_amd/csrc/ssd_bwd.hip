@@ -329,6 +329,21 @@ slice_sum_kernel(const SliceSumArgs a) {
 // Group-level finish: dG = sum of the slice partials; dC = dG B + sum dCoff;  dB = dG^T C + sum dBoff.
 // grid (nchunks, ngroups, batch), 512 threads.  The head-summed dG is rounded to the operand type only here; for
 // bf16 it is split into hi + lo (two MFMA passes) so the contractions see it at ~2^-17 relative.
+// acc[0][j] += A[rows 0..31, k0:k1] * M[column blocks nb0 + j, k0:k1]^T with A in LDS (row-major) and M a transposed
+// B / C tile in MFMA operand order (mt_offset), copied to LDS as it lies: a wave's B-operand fragment is one
+// contiguous KiB.
+template <int NB, typename T>
+__device__ __forceinline__ void wave_mma_mt(floatx16 (&acc)[1][NB], const T* __restrict__ A, int lda, const T* __restrict__ Mt,
+                                            int nb0, int k0, int k1) {
+    const int lane = threadIdx.x & 63;
+    const int r = lane & 31, kh = (lane >> 5) * 8;
+    for (int k = k0; k < k1; k += 16) {
+        const Frag<T> af = load_frag(A + r * lda + k + kh);
+#pragma unroll
+        for (int j = 0; j < NB; ++j) mma_frag(acc[0][j], af, load_frag(Mt + (((nb0 + j) * (kQ / 16) + (k >> 4)) * 64 + lane) * 8));
+    }
+}
+
 template <typename T, int N>
 __global__ void __launch_bounds__(512)
 bc_final_kernel(const float* __restrict__ dGp, const float* __restrict__ dCp, const float* __restrict__ dBp,
@@ -370,7 +385,14 @@ bc_final_kernel(const float* __restrict__ dGp, const float* __restrict__ dCp, co
     }
     constexpr int NPASS = sizeof(T) == 2 ? 2 : 1;
     // dC[i][n] += sum_{j<=i} dG[i][j] B[j][n]
-    stage_rows<T, N, kQ, 512, false>(sT2, LDQ, Bt + grp * (int64_t)(N * kQ), kQ, N, nullptr, tid);
+    auto stage_mt = [&](const T* tile) {
+        if constexpr (sizeof(T) == 2) {
+            for (int e = tid; e < N * kQ / 8; e += 512) *reinterpret_cast<uint4*>(sT2 + e * 8) = *reinterpret_cast<const uint4*>(tile + e * 8);
+        } else {
+            stage_rows<T, N, kQ, 512, false>(sT2, LDQ, tile, kQ, N, nullptr, tid);
+        }
+    };
+    stage_mt(Bt + grp * (int64_t)(N * kQ));
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
 #pragma unroll
@@ -383,11 +405,12 @@ bc_final_kernel(const float* __restrict__ dGp, const float* __restrict__ dCp, co
                 sA2[i * LDQ + j] = pass == 0 ? hi : from_f32<T>(full - to_f32(hi));
             }
         __syncthreads();
-        wave_mma<1, NB>(aC, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, 0, (rb + 1) * 32);
+        if constexpr (sizeof(T) == 2) wave_mma_mt<NB>(aC, sA2 + rb * 32 * LDQ, LDQ, sT2, nb0, 0, (rb + 1) * 32);
+        else wave_mma<1, NB>(aC, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, 0, (rb + 1) * 32);
         __syncthreads();
     }
     // dB[j][n] += sum_{i>=j} dG[i][j] C[i][n]
-    stage_rows<T, N, kQ, 512, false>(sT2, LDQ, Ct + grp * (int64_t)(N * kQ), kQ, N, nullptr, tid);
+    stage_mt(Ct + grp * (int64_t)(N * kQ));
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
 #pragma unroll
@@ -400,7 +423,8 @@ bc_final_kernel(const float* __restrict__ dGp, const float* __restrict__ dCp, co
                 sA2[j * LDQ + i] = pass == 0 ? hi : from_f32<T>(full - to_f32(hi));
             }
         __syncthreads();
-        wave_mma<1, NB>(aB, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, rb * 32, kQ);
+        if constexpr (sizeof(T) == 2) wave_mma_mt<NB>(aB, sA2 + rb * 32 * LDQ, LDQ, sT2, nb0, rb * 32, kQ);
+        else wave_mma<1, NB>(aB, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, rb * 32, kQ);
         __syncthreads();
     }
     T* dBo = dB + b * dBsb + t0 * dBsl + g * dBsg;
@@ -470,8 +494,20 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
     int rc;
     // decay tables, G (+ operand tiles) and the state entering each chunk, unless the caller kept the forward's
     if (!p->chunk_states && (rc = ssd_launch_states<T, P, N>(p, w, nullptr, st))) return rc;
-    // local dS contributions (reuses the `local` region) and the reverse recurrence
-    {
+    // gradient of the state leaving each chunk (reverse recurrence over the chunks' own contributions)
+    if constexpr (sizeof(T) == 2) {
+        auto k = state_pass16_kernel<T, P, N, true>;
+        const size_t sm = state_pass_smem<P, N>();
+        if ((rc = allow_smem(k, sm))) return rc;
+        StatePassArgs sa;
+        sa.X = dy; sa.X_sb = p->dy_stride_b; sa.X_sl = p->dy_stride_l; sa.X_sh = p->dy_stride_h;
+        sa.ldtab = w.ldtab; sa.Mt = w.Ct; sa.init = p->d_final_state; sa.prev = w.dprev; sa.final_out = p->d_initial_state;
+        sa.sprev = w.prev; sa.dlam = w.dlam;
+        sa.seqlen = p->seqlen; sa.nheads = p->nheads; sa.ngroups = p->ngroups; sa.nchunks = nc;
+        k<<<dim3((unsigned)(p->nheads * state_pass_nsplit<N>()), (unsigned)p->batch), 256, sm, st>>>(sa);
+        if ((rc = check_launch("ssd state_pass16_kernel<reverse>"))) return rc;
+    } else
+    {   // fp32: local dS contributions (reuses the `local` region), then the reverse recurrence
         auto dstates = [&](auto lt_tag) -> int {
             using LT = decltype(lt_tag);
             auto k = chunk_state_kernel<T, P, N, true, LT>;

@@ -426,7 +426,7 @@ da_kernel(const float* __restrict__ ldtab, const float* __restrict__ A,
     const float dta = ldtab[bhc * 2 * kQ + kQ + ta], dtb = ldtab[bhc * 2 * kQ + kQ + tb];     // 0 past the end of the sequence
     float dlm = 0.f;
 #pragma unroll
-    for (int sp = 0; sp < kScanSplit; ++sp) dlm += dlam[bhc * kScanSplit + sp];
+    for (int sp = 0; sp < kDlamParts; ++sp) dlm += dlam[bhc * kDlamParts + sp];
     float ya = ra, yb = rbv;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {

@@ -316,7 +316,7 @@ diag_off_kernel(const DiagArgs a) {
                 xb += yb - rbv;
                 float dlm = 0.f;
 #pragma unroll
-                for (int sp = 0; sp < kScanSplit; ++sp) dlm += a.dlam[bhc * kScanSplit + sp];
+                for (int sp = 0; sp < kDlamParts; ++sp) dlm += a.dlam[bhc * kDlamParts + sp];
                 const float da_a = xa + dlm, da_b = xb + dlm;
                 float dAl = 0.f;
                 if (ta < valid) {

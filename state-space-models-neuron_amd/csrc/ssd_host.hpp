@@ -4,6 +4,7 @@
 #include "ssd_diag.hpp"
 #include "ssd_bwd_main.hpp"
 #include "ssd_dg.hpp"
+#include "ssd_states16.hpp"
 
 namespace m2 {
 
@@ -96,7 +97,7 @@ inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd, bool
             w.ns_c = w.ns_b; w.hps_c = w.hps_b;
         }
         w.dprev = take(tiles * esz);
-        w.dlam = reinterpret_cast<float*>(take(bhc * 4 * kScanSplit));
+        w.dlam = reinterpret_cast<float*>(take(bhc * 4 * kDlamParts));
         w.dAp = reinterpret_cast<float*>(take(bhc * 4));
         w.dDp = reinterpret_cast<float*>(take(bhc * 4));
         w.dl = reinterpret_cast<float*>(take(bhc * kQ * 4));
@@ -177,6 +178,19 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
             p->C_stride_b, p->C_stride_l, p->C_stride_g);
         if ((rc = check_launch("ssd cb_kernel"))) return rc;
     }
+    if constexpr (sizeof(T) == 2) {
+        // 16-bit operands: contributions and recurrence in one pass, running state in registers
+        auto k = state_pass16_kernel<T, P, N, false>;
+        const size_t sm = state_pass_smem<P, N>();
+        if ((rc = allow_smem(k, sm))) return rc;
+        StatePassArgs sa;
+        sa.X = x; sa.X_sb = p->x_stride_b; sa.X_sl = p->x_stride_l; sa.X_sh = p->x_stride_h;
+        sa.ldtab = w.ldtab; sa.Mt = w.Bt; sa.init = p->initial_state; sa.prev = w.prev; sa.final_out = final_out;
+        sa.sprev = nullptr; sa.dlam = nullptr;
+        sa.seqlen = p->seqlen; sa.nheads = p->nheads; sa.ngroups = p->ngroups; sa.nchunks = nc;
+        k<<<dim3((unsigned)(p->nheads * state_pass_nsplit<N>()), (unsigned)p->batch), 256, sm, st>>>(sa);
+        return check_launch("ssd state_pass16_kernel");
+    } else {
     // per-chunk contributions in fp32 when an fp32 state leaves the call, otherwise in the operand type
     auto states = [&](auto lt_tag) -> int {
         using LT = decltype(lt_tag);
@@ -199,6 +213,7 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
     else rc = states(T{});
     if (rc) return rc;
     return M2_OK;
+    }
 }
 
 #define M2_DISPATCH_PN(p, P, N, ...)                                                     \

@@ -29,9 +29,21 @@ namespace m2 {
 //   Gf  [kQ][kQ] fp32            G[i][j] (all blocks with block-row >= block-col)
 //   Gm  [kQ][kQ] T               causal G:  G[i][j] for i >= j, else 0         (forward diagonal term, rows i)
 //   Gmt [kQ][kQ] T               its transpose: Gmt[j][i] = G[i][j] for i >= j (backward dx term, rows j)
-//   Bt, Ct [N][kQ] T             B and C transposed (tokens contiguous): MFMA operands of the chunk-state products
+//   Bt, Ct N x kQ T              B and C transposed (tokens contiguous), laid out by mt_offset: MFMA operands of the
+//                                chunk-state products
 // grid (nchunks, ngroups, batch), 256 threads.  The upper-right 64x64 quadrant of G is never consumed and is
 // neither computed nor written.
+// Element offset of the 8 tokens s0 .. s0 + 7 (s0 a multiple of 8) of state column n inside a transposed B / C tile.
+//   fp32   : [N][kQ], tokens contiguous (rows staged into LDS by chunk_state_kernel);
+//   16-bit : MFMA operand order [N / 32][kQ / 16][64 lanes][8]: the B-operand fragment of a wave for column block n / 32
+//            and k-step s0 / 16 is one contiguous KiB, lane = 32 ((s0 / 8) & 1) + n % 32 (read by state_pass16_kernel
+//            straight into registers, eight full cache lines per load instruction).
+template <typename T>
+__device__ __forceinline__ int64_t mt_offset(int n, int s0) {
+    if (sizeof(T) == 2) return ((int64_t)((n >> 5) * (kQ / 16) + (s0 >> 4)) * 64 + ((s0 >> 3) & 1) * 32 + (n & 31)) * 8;
+    return (int64_t)n * kQ + s0;
+}
+
 template <typename T, int N>
 __global__ void __launch_bounds__(256)
 cb_kernel(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict__ Gf, T* __restrict__ Gm, T* __restrict__ Gmt,
@@ -67,8 +79,8 @@ cb_kernel(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict_
             T vb[V], vc[V];
 #pragma unroll
             for (int q = 0; q < V; ++q) { vb[q] = sB[(s0 + q) * LD + n]; vc[q] = sC[(s0 + q) * LD + n]; }
-            *reinterpret_cast<uint4*>(Btp + (int64_t)(k0 + n) * kQ + s0) = *reinterpret_cast<const uint4*>(vb);
-            *reinterpret_cast<uint4*>(Ctp + (int64_t)(k0 + n) * kQ + s0) = *reinterpret_cast<const uint4*>(vc);
+            *reinterpret_cast<uint4*>(Btp + mt_offset<T>(k0 + n, s0)) = *reinterpret_cast<const uint4*>(vb);
+            *reinterpret_cast<uint4*>(Ctp + mt_offset<T>(k0 + n, s0)) = *reinterpret_cast<const uint4*>(vc);
         }
         __syncthreads();
     }
@@ -242,6 +254,7 @@ chunk_state_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
 // subtracting a suffix sum there would cancel two large numbers rounded differently (operand-type copies of
 // the states), leaving an error that is constant over the chunk and accumulates in dA.
 constexpr int kScanSplit = 4;
+constexpr int kDlamParts = 8;     // partial sums of dlam per (batch, head, chunk): every producer fills all of them
 
 template <typename T, int PN, bool REVERSE, typename LT>
 __global__ void __launch_bounds__(256)
@@ -301,7 +314,10 @@ state_scan_kernel(const LT* __restrict__ local, const float* __restrict__ lam, c
                 const int64_t first = cc - (cc % kRedBatch);
                 if (tid <= cc - first) {
                     const int64_t c2 = REVERSE ? nchunks - 1 - (first + tid) : first + tid;
-                    dlam[(bh * nchunks + c2) * kScanSplit + blockIdx.z] = red[tid * 4] + red[tid * 4 + 1] + red[tid * 4 + 2] + red[tid * 4 + 3];
+                    {
+                        dlam[(bh * nchunks + c2) * kDlamParts + blockIdx.z] = red[tid * 4] + red[tid * 4 + 1] + red[tid * 4 + 2] + red[tid * 4 + 3];
+                        dlam[(bh * nchunks + c2) * kDlamParts + kScanSplit + blockIdx.z] = 0.f;
+                    }
                 }
                 __syncthreads();
             }

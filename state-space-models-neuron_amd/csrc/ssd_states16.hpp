@@ -1,0 +1,255 @@
+// Chunk states for 16-bit operands in ONE pass: the per-chunk contributions and the recurrence over the chunks fused,
+// with the running state in registers (fp32), so that no per-chunk contribution is ever written to memory.
+//
+//   forward:  S = init;   for c = 0 .. nc-1:   prev[c] = T(S);   S = e^{Lam_c} S + sum_j (dt_j e^{Lam_c - l_j}) x_j (x) B_j;   final = S
+//   reverse:  R = dfinal; for c = nc-1 .. 0:   prev[c] = T(R);   dlam[c] = e^{Lam_c} <T(R), sprev[c]>;
+//                                              R = e^{Lam_c} R + sum_i e^{l_i} dy_i (x) C_i;   dinit = R
+// (dlam is the part of dL/dLam_c that flows through the carried state; sprev[c] = the forward state entering chunk c.)
+//
+// grid (nheads * NSPLIT, batch), 4 waves; a workgroup owns N / NSPLIT columns of the [P][N] state, wave w rows
+// [ (w & 1) P/2, +P/2 ) x half of those columns, as 32x32 MFMA accumulator blocks.  Per chunk the MFMA computes  X_scaled^T [P x kQ] * M [kQ x N]:
+//   * M (B or C of the group) comes from the transposed tiles that cb_kernel wrote in MFMA operand order: a wave's
+//     B-operand fragment is one contiguous KiB of global memory, loaded straight into registers at the top of the
+//     chunk's iteration (the tile is shared by all heads of the group and stays in L2);
+//   * x / dy rows are loaded one chunk ahead into registers, scaled per token in fp32, rounded once and written
+//     row-major into one of two LDS buffers (one barrier per chunk); the A-operand fragments (k = token contiguous)
+//     come out of it through LDS transpose reads.
+// The state leaves through a wave-private LDS tile so that each lane stores 16 contiguous bytes of a state row.
+#pragma once
+#include "ssd_y.hpp"
+
+namespace m2 {
+
+// the two 16-bit elements of a 32-bit word as fp32, and back (round to nearest even)
+template <typename T> __device__ __forceinline__ float unpack_lo(uint32_t w);
+template <typename T> __device__ __forceinline__ float unpack_hi(uint32_t w);
+template <> __device__ __forceinline__ float unpack_lo<bf16_t>(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+template <> __device__ __forceinline__ float unpack_hi<bf16_t>(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef T tvec2 __attribute__((ext_vector_type(2)));
+    const tvec2 v = {from_f32<T>(lo), from_f32<T>(hi)};
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+struct StatePassArgs {
+    const void* X; int64_t X_sb, X_sl, X_sh;      // x (forward) / dy (reverse): [b][l][h][P]
+    const float* ldtab;                            // [b][h][c][ l kQ | dt kQ ]
+    const void* Mt;                                // B^T (forward) / C^T (reverse) tiles: [b][c][g][N x kQ in operand order]
+    const float* init;                             // fp32 [b][h][P][N]: initial state / gradient of the final state, or null
+    void* prev;                                    // out [b][c][h][P][N], operand type
+    float* final_out;                              // out fp32 [b][h][P][N]: final state / gradient of the initial state, or null
+    const void* sprev;                             // reverse: [b][c][h][P][N] forward states entering the chunks
+    float* dlam;                                   // reverse: out [b][h][c][kDlamParts]
+    int64_t seqlen, nheads, ngroups, nchunks;
+};
+
+// workgroups per (batch, head): each takes N / NSPLIT state columns (more, smaller workgroups: the chunk loop is a
+// chain of dependent memory round trips, and only other resident waves can fill its gaps)
+template <int N> constexpr int state_pass_nsplit() { return N / 64; }
+template <int P, int N>
+constexpr size_t state_pass_smem() { return (size_t)2 * kQ * P * 2 + (size_t)4 * (P / 2) * (N / state_pass_nsplit<N>() / 2 + 8) * 2; }
+
+template <typename T, int P, int N, bool REVERSE>
+__global__ void __launch_bounds__(256, 2)
+state_pass16_kernel(const StatePassArgs a) {
+    static_assert(sizeof(T) == 2, "16-bit operands only");
+    constexpr int NSPLIT = state_pass_nsplit<N>();
+    constexpr int NW = N / NSPLIT / 2;                 // state columns per wave
+    constexpr int PBW = P / 64, NBW = NW / 32;         // 32x32 blocks per wave
+    constexpr int SPR_X = P / 8;                       // 16-byte slots per x row
+    constexpr int NXR = kQ * SPR_X / 256;              // x pieces per thread per chunk
+    constexpr int LDO = NW + 8;
+    constexpr int LPR = NW / 8;                   // lanes per row of this wave's state block (8 elements each)
+    constexpr int RPP = 64 / LPR;                      // rows per store pass
+    constexpr int NSP = (P / 2) / RPP;                 // store passes
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* sX = reinterpret_cast<T*>(smem_raw);                                 // [2][kQ][P], slots swizzled inside each row
+    T* sO = sX + 2 * kQ * P;                                                // [4 waves][P / 2][LDO]
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 31, half = lane >> 5;
+    const int pw = wave & 1, nw = wave >> 1;
+    // the workgroups of one head are nheads apart in the grid: with a head count that is a multiple of 8 they land on the
+    // same XCD and share the head's rows in its L2
+    const int64_t h = blockIdx.x % a.nheads, b = blockIdx.y;
+    const int n0 = (int)(blockIdx.x / a.nheads) * (N / NSPLIT) + nw * NW;      // first state column of this wave
+    const int64_t g = h / (a.nheads / a.ngroups);
+    const int64_t bh = b * a.nheads + h;
+    const int64_t nc = a.nchunks;
+    T* sOw = sO + wave * (P / 2) * LDO;
+    const int tr_tok = 8 * half + ((lane >> 2) & 3);
+    const int tr_col = ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+    typedef T tvec4 __attribute__((ext_vector_type(4)));
+
+    floatx16 acc[PBW][NBW];
+#pragma unroll
+    for (int i = 0; i < PBW; ++i)
+#pragma unroll
+        for (int j = 0; j < NBW; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = pw * (P / 2) + i * 32 + acc_row(lane, v), col = n0 + j * 32 + r;
+                acc[i][j][v] = a.init ? a.init[bh * (P * N) + row * N + col] : 0.f;
+            }
+
+    // two chunks ahead in registers, in two sets used alternately: the x / dy pieces with their token's l and dt, and
+    // the chunk's Lam.  The values of chunk cc are consumed before the barrier of its iteration; behind it the same set
+    // is loaded with chunk cc + 2, so that a load has two iterations to land.
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    struct Ahead { u32x4 x[NXR]; float l[NXR], d[NXR], lam; };
+    auto chunk_of = [&](int64_t cc) -> int64_t {       // cc-th chunk in processing order, clamped to the last one
+        const int64_t k = cc < nc ? cc : nc - 1;
+        return REVERSE ? nc - 1 - k : k;
+    };
+    auto load_ahead = [&](int64_t c, Ahead& s) {
+        const int64_t t0 = c * kQ;
+        const int valid = (int)((a.seqlen - t0) < kQ ? (a.seqlen - t0) : kQ);
+        const T* xp = static_cast<const T*>(a.X) + b * a.X_sb + t0 * a.X_sl + h * a.X_sh;
+        const float* tab = a.ldtab + (bh * nc + c) * (2 * kQ);
+        s.lam = tab[kQ - 1];
+#pragma unroll
+        for (int it = 0; it < NXR; ++it) {
+            const int e = it * 256 + tid, row = e / SPR_X, slot = e % SPR_X;
+            const int grow = row < valid ? row : valid - 1;      // rows past the end: finite stand-ins, scaled by zero
+            s.x[it] = *reinterpret_cast<const u32x4*>(xp + (int64_t)grow * a.X_sl + slot * 8);
+            s.l[it] = tab[row];
+            s.d[it] = REVERSE ? (row < valid ? 1.f : 0.f) : tab[kQ + row];      // dt is 0 past the end of the sequence
+        }
+    };
+    // loaded at the top of the iteration that consumes them (so that the wait in front of their use can be counted
+    // exactly and leaves the next chunk's rows, issued behind them, in flight): the group's B^T / C^T fragments (L2) and,
+    // for the reverse pass, this lane's pieces of the forward state
+    Frag<T> bf[NBW][8];
+    u32x4 spr[REVERSE ? NSP : 1];
+    auto load_same = [&](int64_t c) {
+        const T* mp = static_cast<const T*>(a.Mt) + ((b * nc + c) * a.ngroups + g) * (int64_t)(N * kQ);
+#pragma unroll
+        for (int j = 0; j < NBW; ++j)
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) bf[j][ks] = load_frag(mp + (((n0 >> 5) + j) * 8 + ks) * 512 + lane * 8);      // see mt_offset
+        if (REVERSE) {
+            const T* sp = static_cast<const T*>(a.sprev) + ((b * nc + c) * a.nheads + h) * (int64_t)(P * N);
+#pragma unroll
+            for (int ps = 0; ps < NSP; ++ps) {
+                const int rl = ps * RPP + lane / LPR, cv = lane % LPR;
+                spr[ps] = *reinterpret_cast<const u32x4*>(sp + (pw * (P / 2) + rl) * N + n0 + cv * 8);
+            }
+        }
+    };
+
+    auto step = [&](int64_t cc, Ahead& s) {
+        const int64_t c = chunk_of(cc);
+        const int buf = (int)(cc & 1);
+        T* cX = sX + buf * (kQ * P);
+        load_same(c);
+        // the values loaded one chunk ahead become visible to the optimiser here and no earlier: otherwise their
+        // unpacking is scheduled right behind the loads, which then wait for the data a whole chunk too early
+#pragma unroll
+        for (int it = 0; it < NXR; ++it)
+            asm volatile("" : "+v"(s.x[it]), "+v"(s.l[it]), "+v"(s.d[it]));      // whole 128-bit vectors: no re-packing
+        asm volatile("" : "+v"(s.lam));
+        // ---- scaled rows into LDS
+#pragma unroll
+        for (int it = 0; it < NXR; ++it) {
+            const int e = it * 256 + tid, row = e / SPR_X, slot = e % SPR_X;
+            const float sc = REVERSE ? s.d[it] * __expf(s.l[it]) : s.d[it] * __expf(s.lam - s.l[it]);
+            // word-wise (two elements per 32-bit word), so that the loaded vectors stay four whole registers until here
+            u32x4 o;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) o[q] = pack2<T>(unpack_lo<T>(s.x[it][q]) * sc, unpack_hi<T>(s.x[it][q]) * sc);
+            *reinterpret_cast<u32x4*>(cX + (row * SPR_X + (slot ^ tile_swz<SPR_X>(row))) * 8) = o;
+        }
+        const float dec = __expf(s.lam);
+        __syncthreads();          // the tile is complete; every wave is done with the other buffer
+        // the rows two chunks on (past the end: the last chunk once more, rather than branching around the loads)
+        load_ahead(chunk_of(cc + 2), s);
+
+        // ---- the state entering (forward) / the gradient leaving (reverse) this chunk, through the wave-private tile
+#pragma unroll
+        for (int i = 0; i < PBW; ++i)
+#pragma unroll
+            for (int j = 0; j < NBW; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) sOw[(i * 32 + acc_row(lane, v)) * LDO + j * 32 + r] = from_f32<T>(acc[i][j][v]);
+        wave_lds_sync();
+        T* op = static_cast<T*>(a.prev) + ((b * nc + c) * a.nheads + h) * (int64_t)(P * N);
+        float dot = 0.f;
+#pragma unroll
+        for (int ps = 0; ps < NSP; ++ps) {
+            const int rl = ps * RPP + lane / LPR, cv = lane % LPR;
+            const u32x4 o = *reinterpret_cast<const u32x4*>(sOw + rl * LDO + cv * 8);
+            *reinterpret_cast<u32x4*>(op + (pw * (P / 2) + rl) * N + n0 + cv * 8) = o;
+            if (REVERSE) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    dot += unpack_lo<T>(o[q]) * unpack_lo<T>(spr[ps][q]) + unpack_hi<T>(o[q]) * unpack_hi<T>(spr[ps][q]);
+            }
+        }
+        if (REVERSE) {
+            dot = warp_sum(dot);
+            if (lane == 0) {
+                const int slot = (int)(blockIdx.x / a.nheads) * 4 + wave;
+                a.dlam[(bh * nc + c) * kDlamParts + slot] = dec * dot;
+                if (NSPLIT == 1) a.dlam[(bh * nc + c) * kDlamParts + 4 + slot] = 0.f;
+            }
+        }
+        wave_lds_sync();
+
+        // ---- S = e^{Lam} S + X_scaled^T M
+#pragma unroll
+        for (int i = 0; i < PBW; ++i)
+#pragma unroll
+            for (int j = 0; j < NBW; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] *= dec;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            const int ta = ks * 16 + tr_tok, tb = ta + 4;
+#pragma unroll
+            for (int i = 0; i < PBW; ++i) {
+                const int col = pw * (P / 2) + i * 32 + tr_col;
+                const tvec4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                    (M2_LDS tvec4*)(cX + (ta * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(ta))) * 8 + (col & 7)));
+                const tvec4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                    (M2_LDS tvec4*)(cX + (tb * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(tb))) * 8 + (col & 7)));
+                Frag<T> af;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { af.v[e] = lo[e]; af.v[4 + e] = hi[e]; }
+#pragma unroll
+                for (int j = 0; j < NBW; ++j) mma_frag(acc[i][j], af, bf[j][ks]);
+            }
+        }
+    };
+
+    // Chunks are taken two per loop iteration (one per register set); an odd first chunk is peeled off in front so that
+    // the loop body is free of conditionals (a branch around loads costs register copies, and with them early waits).
+    Ahead s0, s1;
+    int64_t cc = 0;
+    if (nc & 1) {
+        load_ahead(chunk_of(0), s1);
+        load_ahead(chunk_of(1), s0);
+        step(0, s1);
+        cc = 1;
+    } else {
+        load_ahead(chunk_of(0), s0);
+        load_ahead(chunk_of(1), s1);
+    }
+#pragma unroll 1
+    for (; cc < nc; cc += 2) {
+        step(cc, s0);
+        step(cc + 1, s1);
+    }
+    if (a.final_out) {
+#pragma unroll
+        for (int i = 0; i < PBW; ++i)
+#pragma unroll
+            for (int j = 0; j < NBW; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = pw * (P / 2) + i * 32 + acc_row(lane, v), col = n0 + j * 32 + r;
+                    a.final_out[bh * (P * N) + row * N + col] = acc[i][j][v];
+                }
+    }
+}
+
+}  // namespace m2
