@@ -6,8 +6,8 @@
 //                                              R = e^{Lam_c} R + sum_i e^{l_i} dy_i (x) C_i;   dinit = R
 // (dlam is the part of dL/dLam_c that flows through the carried state; sprev[c] = the forward state entering chunk c.)
 //
-// grid (nheads * NSPLIT, batch), 4 waves; a workgroup owns N / NSPLIT columns of the [P][N] state, wave w rows
-// [ (w & 1) P/2, +P/2 ) x half of those columns, as 32x32 MFMA accumulator blocks.  Per chunk the MFMA computes  X_scaled^T [P x kQ] * M [kQ x N]:
+// grid (nheads * NSPLIT, batch), 2 x NWG waves; a workgroup owns N / NSPLIT columns of the [P][N] state, wave w rows
+// [ (w & 1) P/2, +P/2 ) x one NWG-th of those columns, as 32x32 MFMA accumulator blocks.  Per chunk the MFMA computes  X_scaled^T [P x kQ] * M [kQ x N]:
 //   * M (B or C of the group) comes from the transposed tiles that cb_kernel wrote in MFMA operand order: a wave's
 //     B-operand fragment is one contiguous KiB of global memory, loaded straight into registers at the top of the
 //     chunk's iteration (the tile is shared by all heads of the group and stays in L2);
@@ -45,26 +45,39 @@ struct StatePassArgs {
 
 // workgroups per (batch, head): each takes N / NSPLIT state columns (more, smaller workgroups: the chunk loop is a
 // chain of dependent memory round trips, and only other resident waves can fill its gaps)
-template <int N> constexpr int state_pass_nsplit() { return N / 64; }
+#ifndef M2_SP_NSPLIT
+#define M2_SP_NSPLIT(N) ((N) / 64)
+#endif
+#ifndef M2_SP_NWG
+#define M2_SP_NWG(N) 2
+#endif
+template <int N> constexpr int state_pass_nsplit() { return M2_SP_NSPLIT(N); }
+// waves per workgroup along the state columns (times two along the rows)
+template <int N> constexpr int state_pass_nwg() { return M2_SP_NWG(N); }
+template <int N> constexpr int state_pass_threads() { return 2 * state_pass_nwg<N>() * 64; }
 template <int P, int N>
-constexpr size_t state_pass_smem() { return (size_t)2 * kQ * P * 2 + (size_t)4 * (P / 2) * (N / state_pass_nsplit<N>() / 2 + 8) * 2; }
+constexpr size_t state_pass_smem() {
+    return (size_t)2 * kQ * P * 2 + (size_t)2 * state_pass_nwg<N>() * (P / 2) * (N / state_pass_nsplit<N>() / state_pass_nwg<N>() + 8) * 2;
+}
 
 template <typename T, int P, int N, bool REVERSE>
-__global__ void __launch_bounds__(256, 2)
+__global__ void __launch_bounds__(state_pass_threads<N>(), (P == 64 ? (REVERSE ? 2 : 3) : (REVERSE ? 1 : 2)))
 state_pass16_kernel(const StatePassArgs a) {
     static_assert(sizeof(T) == 2, "16-bit operands only");
     constexpr int NSPLIT = state_pass_nsplit<N>();
-    constexpr int NW = N / NSPLIT / 2;                 // state columns per wave
+    constexpr int NWG = state_pass_nwg<N>(), THREADS = state_pass_threads<N>();
+    constexpr int NW = N / NSPLIT / NWG;               // state columns per wave
+    static_assert(NW % 32 == 0 && 2 * NWG * NSPLIT <= kDlamParts, "wave blocks / dlam slots");
     constexpr int PBW = P / 64, NBW = NW / 32;         // 32x32 blocks per wave
     constexpr int SPR_X = P / 8;                       // 16-byte slots per x row
-    constexpr int NXR = kQ * SPR_X / 256;              // x pieces per thread per chunk
+    constexpr int NXR = kQ * SPR_X / THREADS;              // x pieces per thread per chunk
     constexpr int LDO = NW + 8;
     constexpr int LPR = NW / 8;                   // lanes per row of this wave's state block (8 elements each)
     constexpr int RPP = 64 / LPR;                      // rows per store pass
     constexpr int NSP = (P / 2) / RPP;                 // store passes
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* sX = reinterpret_cast<T*>(smem_raw);                                 // [2][kQ][P], slots swizzled inside each row
-    T* sO = sX + 2 * kQ * P;                                                // [4 waves][P / 2][LDO]
+    T* sO = sX + 2 * kQ * P;                                                // [waves][P / 2][LDO]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 31, half = lane >> 5;
@@ -101,19 +114,24 @@ state_pass16_kernel(const StatePassArgs a) {
         const int64_t k = cc < nc ? cc : nc - 1;
         return REVERSE ? nc - 1 - k : k;
     };
+    // Addresses are a wave-uniform base (scalar registers) plus a 32-bit per-lane byte offset, recomputed from the thread
+    // index where it is cheap: 64-bit per-lane pointers kept alive across the chunk loop cost more registers than the data.
+    const uint32_t row_t = (uint32_t)tid / SPR_X, slot_t = (uint32_t)tid % SPR_X;      // piece `it` of this thread: row_t + it * RSTEP
+    constexpr int RSTEP = THREADS / SPR_X;
+    const uint32_t x_row_bytes = (uint32_t)(a.X_sl * 2);
     auto load_ahead = [&](int64_t c, Ahead& s) {
         const int64_t t0 = c * kQ;
-        const int valid = (int)((a.seqlen - t0) < kQ ? (a.seqlen - t0) : kQ);
-        const T* xp = static_cast<const T*>(a.X) + b * a.X_sb + t0 * a.X_sl + h * a.X_sh;
+        const uint32_t last = (uint32_t)(((a.seqlen - t0) < kQ ? (a.seqlen - t0) : kQ) - 1);      // last valid row
+        const char* xp = reinterpret_cast<const char*>(static_cast<const T*>(a.X) + b * a.X_sb + t0 * a.X_sl + h * a.X_sh);
         const float* tab = a.ldtab + (bh * nc + c) * (2 * kQ);
         s.lam = tab[kQ - 1];
 #pragma unroll
         for (int it = 0; it < NXR; ++it) {
-            const int e = it * 256 + tid, row = e / SPR_X, slot = e % SPR_X;
-            const int grow = row < valid ? row : valid - 1;      // rows past the end: finite stand-ins, scaled by zero
-            s.x[it] = *reinterpret_cast<const u32x4*>(xp + (int64_t)grow * a.X_sl + slot * 8);
+            const uint32_t row = row_t + it * RSTEP;
+            const uint32_t grow = row < last ? row : last;      // rows past the end: finite stand-ins, scaled by zero
+            s.x[it] = *reinterpret_cast<const u32x4*>(xp + (grow * x_row_bytes + slot_t * 16u));
             s.l[it] = tab[row];
-            s.d[it] = REVERSE ? (row < valid ? 1.f : 0.f) : tab[kQ + row];      // dt is 0 past the end of the sequence
+            s.d[it] = REVERSE ? (row <= last ? 1.f : 0.f) : tab[kQ + row];      // dt is 0 past the end of the sequence
         }
     };
     // loaded at the top of the iteration that consumes them (so that the wait in front of their use can be counted
@@ -121,19 +139,18 @@ state_pass16_kernel(const StatePassArgs a) {
     // for the reverse pass, this lane's pieces of the forward state
     Frag<T> bf[NBW][8];
     u32x4 spr[REVERSE ? NSP : 1];
+    const uint32_t st_off = (uint32_t)(((pw * (P / 2) + lane / LPR) * N + n0 + (lane % LPR) * 8) * 2);      // pass ps: + ps * RPP * N * 2
     auto load_same = [&](int64_t c) {
-        const T* mp = static_cast<const T*>(a.Mt) + ((b * nc + c) * a.ngroups + g) * (int64_t)(N * kQ);
+        const char* mp = reinterpret_cast<const char*>(static_cast<const T*>(a.Mt) + ((b * nc + c) * a.ngroups + g) * (int64_t)(N * kQ));
 #pragma unroll
         for (int j = 0; j < NBW; ++j)
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) bf[j][ks] = load_frag(mp + (((n0 >> 5) + j) * 8 + ks) * 512 + lane * 8);      // see mt_offset
+            for (int ks = 0; ks < 8; ++ks)      // see mt_offset
+                bf[j][ks].v = *reinterpret_cast<const bf16x8*>(mp + ((uint32_t)lane * 16u + (uint32_t)((((n0 >> 5) + j) * 8 + ks) * 1024)));
         if (REVERSE) {
-            const T* sp = static_cast<const T*>(a.sprev) + ((b * nc + c) * a.nheads + h) * (int64_t)(P * N);
+            const char* sp = reinterpret_cast<const char*>(static_cast<const T*>(a.sprev) + ((b * nc + c) * a.nheads + h) * (int64_t)(P * N));
 #pragma unroll
-            for (int ps = 0; ps < NSP; ++ps) {
-                const int rl = ps * RPP + lane / LPR, cv = lane % LPR;
-                spr[ps] = *reinterpret_cast<const u32x4*>(sp + (pw * (P / 2) + rl) * N + n0 + cv * 8);
-            }
+            for (int ps = 0; ps < NSP; ++ps) spr[ps] = *reinterpret_cast<const u32x4*>(sp + (st_off + (uint32_t)(ps * RPP * N * 2)));
         }
     };
 
@@ -141,6 +158,7 @@ state_pass16_kernel(const StatePassArgs a) {
         const int64_t c = chunk_of(cc);
         const int buf = (int)(cc & 1);
         T* cX = sX + buf * (kQ * P);
+        __builtin_amdgcn_sched_barrier(0);      // keep this chunk's loads out of the previous chunk's MFMA phase (registers)
         load_same(c);
         // the values loaded one chunk ahead become visible to the optimiser here and no earlier: otherwise their
         // unpacking is scheduled right behind the loads, which then wait for the data a whole chunk too early
@@ -151,7 +169,7 @@ state_pass16_kernel(const StatePassArgs a) {
         // ---- scaled rows into LDS
 #pragma unroll
         for (int it = 0; it < NXR; ++it) {
-            const int e = it * 256 + tid, row = e / SPR_X, slot = e % SPR_X;
+            const int row = (int)row_t + it * RSTEP, slot = (int)slot_t;
             const float sc = REVERSE ? s.d[it] * __expf(s.l[it]) : s.d[it] * __expf(s.lam - s.l[it]);
             // word-wise (two elements per 32-bit word), so that the loaded vectors stay four whole registers until here
             u32x4 o;
@@ -172,13 +190,13 @@ state_pass16_kernel(const StatePassArgs a) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) sOw[(i * 32 + acc_row(lane, v)) * LDO + j * 32 + r] = from_f32<T>(acc[i][j][v]);
         wave_lds_sync();
-        T* op = static_cast<T*>(a.prev) + ((b * nc + c) * a.nheads + h) * (int64_t)(P * N);
+        char* op = reinterpret_cast<char*>(static_cast<T*>(a.prev) + ((b * nc + c) * a.nheads + h) * (int64_t)(P * N));
         float dot = 0.f;
 #pragma unroll
         for (int ps = 0; ps < NSP; ++ps) {
             const int rl = ps * RPP + lane / LPR, cv = lane % LPR;
             const u32x4 o = *reinterpret_cast<const u32x4*>(sOw + rl * LDO + cv * 8);
-            *reinterpret_cast<u32x4*>(op + (pw * (P / 2) + rl) * N + n0 + cv * 8) = o;
+            *reinterpret_cast<u32x4*>(op + (st_off + (uint32_t)(ps * RPP * N * 2))) = o;
             if (REVERSE) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
@@ -188,9 +206,9 @@ state_pass16_kernel(const StatePassArgs a) {
         if (REVERSE) {
             dot = warp_sum(dot);
             if (lane == 0) {
-                const int slot = (int)(blockIdx.x / a.nheads) * 4 + wave;
+                const int slot = (int)(blockIdx.x / a.nheads) * (2 * NWG) + wave;
                 a.dlam[(bh * nc + c) * kDlamParts + slot] = dec * dot;
-                if (NSPLIT == 1) a.dlam[(bh * nc + c) * kDlamParts + 4 + slot] = 0.f;
+                if (2 * NWG * NSPLIT < kDlamParts && slot + 2 * NWG * NSPLIT < kDlamParts) a.dlam[(bh * nc + c) * kDlamParts + slot + 2 * NWG * NSPLIT] = 0.f;
             }
         }
         wave_lds_sync();
