@@ -508,27 +508,19 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         if ((rc = check_launch("ssd state_pass16_kernel<reverse>"))) return rc;
     } else
     {   // fp32: local dS contributions (reuses the `local` region), then the reverse recurrence
-        auto dstates = [&](auto lt_tag) -> int {
-            using LT = decltype(lt_tag);
-            auto k = chunk_state_kernel<T, P, N, true, LT>;
-            const size_t sm = state_smem<T, P, N, LT>();
-            int rc2;
-            if ((rc2 = allow_smem(k, sm))) return rc2;
-            int64_t ns, hps;
-            ssd_slicing(p, kWgsChunkState, &ns, &hps);
-            k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * ns), (unsigned)p->batch), 256, sm, st>>>(
-                dy, w.ldtab, static_cast<const T*>(w.Ct), reinterpret_cast<LT*>(w.local), p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
-                p->dy_stride_b, p->dy_stride_l, p->dy_stride_h);
-            if ((rc2 = check_launch("ssd chunk_state_kernel<dstate>"))) return rc2;
-            state_scan_kernel<T, P * N, true, LT><<<dim3((unsigned)p->nheads, (unsigned)p->batch, kScanSplit), 256, 0, st>>>(
-                reinterpret_cast<const LT*>(w.local), w.lam, p->d_final_state, static_cast<T*>(w.dprev), p->d_initial_state,
-                static_cast<const T*>(w.prev), w.dlam, p->nheads, nc);
-            return check_launch("ssd state_scan_kernel<reverse>");
-        };
-        // fp32 contributions when the gradient of the initial state (an fp32 state) leaves the call
-        if (p->d_initial_state) rc = dstates(float{});
-        else rc = dstates(T{});
-        if (rc) return rc;
+        auto k = chunk_state_kernel<T, P, N, true>;
+        const size_t sm = state_smem<T, P, N>();
+        if ((rc = allow_smem(k, sm))) return rc;
+        int64_t ns, hps;
+        ssd_slicing(p, kWgsChunkState, &ns, &hps);
+        k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * ns), (unsigned)p->batch), 256, sm, st>>>(
+            dy, w.ldtab, static_cast<const T*>(w.Ct), w.local, p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
+            p->dy_stride_b, p->dy_stride_l, p->dy_stride_h);
+        if ((rc = check_launch("ssd chunk_state_kernel<dstate>"))) return rc;
+        state_scan_kernel<T, P * N, true><<<dim3((unsigned)p->nheads, (unsigned)p->batch, kScanSplit), 256, 0, st>>>(
+            w.local, w.lam, p->d_final_state, static_cast<T*>(w.dprev), p->d_initial_state,
+            static_cast<const T*>(w.prev), w.dlam, p->nheads, nc);
+        if ((rc = check_launch("ssd state_scan_kernel<reverse>"))) return rc;
     }
     {
         if constexpr (sizeof(T) == 2 && dg16_smem<P>() <= 160 * 1024) {

@@ -64,7 +64,8 @@ inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd, bool
     SsdWorkspace w;
     unsigned char* b8 = static_cast<unsigned char*>(base);
     auto take = [&](size_t n) { unsigned char* r = b8 ? b8 + off : nullptr; off += align_up(n, 256); return r; };
-    w.local = reinterpret_cast<float*>(take(tiles * 4));
+    // per-chunk state contributions: only the fp32 path materialises them (16-bit operands take the fused state pass)
+    if (p->dtype == M2_F32) w.local = reinterpret_cast<float*>(take(tiles * 4));
     // What the backward reuses from the forward: the state entering each chunk, the decay tables and the
     // per-(chunk, group) operand tiles.  They live in the caller's chunk_states buffer when one is given
     // (forward writes, backward reads), otherwise in the workspace (backward recomputes them).
@@ -148,8 +149,8 @@ inline int allow_smem(K kernel, size_t bytes) {
     return M2_OK;
 }
 
-template <typename T, int P, int N, typename LT>
-inline size_t state_smem() { return (size_t)(P + N) * lds_ld<T>(kQ) * sizeof(T) + (sizeof(LT) == 2 ? (size_t)4 * (P / 2) * (N / 2 + 8) * 2 : 0); }
+template <typename T, int P, int N>
+inline size_t state_smem() { return (size_t)(P + N) * lds_ld<T>(kQ) * sizeof(T); }
 template <typename T>
 inline size_t cb_smem() { return (size_t)2 * kQ * lds_ld<T>(64) * sizeof(T); }
 
@@ -191,28 +192,21 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
         k<<<dim3((unsigned)(p->nheads * state_pass_nsplit<N>()), (unsigned)p->batch), state_pass_threads<N>(), sm, st>>>(sa);
         return check_launch("ssd state_pass16_kernel");
     } else {
-    // per-chunk contributions in fp32 when an fp32 state leaves the call, otherwise in the operand type
-    auto states = [&](auto lt_tag) -> int {
-        using LT = decltype(lt_tag);
-        auto k = chunk_state_kernel<T, P, N, false, LT>;
-        const size_t sm = state_smem<T, P, N, LT>();
-        int rc2;
-        if ((rc2 = allow_smem(k, sm))) return rc2;
+        // fp32 operands: per-chunk contributions (fp32, workspace), then the recurrence over the chunks
+        auto k = chunk_state_kernel<T, P, N, false>;
+        const size_t sm = state_smem<T, P, N>();
+        if ((rc = allow_smem(k, sm))) return rc;
         int64_t ns, hps;
         ssd_slicing(p, kWgsChunkState, &ns, &hps);
         M2_REQUIRE(p->ngroups * ns <= 65535, M2_ERR_SHAPE, "ssd: too many group slices");
         k<<<dim3((unsigned)nc, (unsigned)(p->ngroups * ns), (unsigned)p->batch), 256, sm, st>>>(
-            x, w.ldtab, static_cast<const T*>(w.Bt), reinterpret_cast<LT*>(w.local), p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
+            x, w.ldtab, static_cast<const T*>(w.Bt), w.local, p->seqlen, p->nheads, p->ngroups, nc, ns, hps,
             p->x_stride_b, p->x_stride_l, p->x_stride_h);
-        if ((rc2 = check_launch("ssd chunk_state_kernel"))) return rc2;
-        state_scan_kernel<T, P * N, false, LT><<<dim3((unsigned)p->nheads, (unsigned)p->batch, kScanSplit), 256, 0, st>>>(
-            reinterpret_cast<const LT*>(w.local), w.lam, p->initial_state, static_cast<T*>(w.prev), final_out, nullptr, nullptr, p->nheads, nc);
-        return check_launch("ssd state_scan_kernel");
-    };
-    if (final_out) rc = states(float{});
-    else rc = states(T{});
-    if (rc) return rc;
-    return M2_OK;
+        if ((rc = check_launch("ssd chunk_state_kernel"))) return rc;
+        state_scan_kernel<T, P * N, false><<<dim3((unsigned)p->nheads, (unsigned)p->batch, kScanSplit), 256, 0, st>>>(
+            w.local, w.lam, p->initial_state, static_cast<T*>(w.prev), final_out, nullptr, nullptr, p->nheads, nc);
+        if ((rc = check_launch("ssd state_scan_kernel"))) return rc;
+        return M2_OK;
     }
 }
 

@@ -18,6 +18,7 @@
 //   state_scan_kernel  sequential-in-chunks, parallel-in-(b,h,p,n) fp32 recurrence; writes the
 //                      state ENTERING each chunk in the MFMA operand type, and the final state
 //                      (REVERSE variant: gradient recurrence + <dS, S> per chunk)
+// The last two serve fp32 operands; for 16-bit operands ssd_states16.hpp does both in one pass.
 #pragma once
 #include "mma.hpp"
 
@@ -138,16 +139,14 @@ ld_table_kernel(const void* __restrict__ dt, int dt_f32, const float* __restrict
 // Local chunk state.  grid (nchunks, ngroups * nslices, batch), 256 threads; a workgroup loops over `hps` heads.
 //   DSTATE == false:  out[p][n] = sum_j (dt_j e^{Lam-l_j}) x[j][p] * B[j][n]      (forward)
 //   DSTATE == true :  out[p][n] = sum_i e^{l_i} dy[i][p] * C[i][n]                (backward)
-// `out` is stored as LT: fp32, or -- for 16-bit operands when no fp32 state leaves the call (no final state / no
-// gradient of the initial state requested) -- the operand type, which halves the traffic of this kernel's output
-// and of the scan's input; the scan itself always accumulates in fp32.
+// Used for fp32 operands (16-bit operands take state_pass16_kernel, which fuses this with the recurrence); `out` is fp32.
 // `X` is x or dy; `Mt` is the group's B or C tile already transposed to [N][kQ] (tokens contiguous) by cb_kernel,
 // staged into LDS once per workgroup.  Per head only the x tile moves: it is loaded 16 bytes at a time, scaled in
 // fp32 and written transposed; the next head's tile is prefetched into registers while the MFMAs run.
-template <typename T, int P, int N, bool DSTATE, typename LT>
+template <typename T, int P, int N, bool DSTATE>
 __global__ void __launch_bounds__(256)
 chunk_state_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
-                   const T* __restrict__ Mt, LT* __restrict__ out,
+                   const T* __restrict__ Mt, float* __restrict__ out,
                    int64_t seqlen, int64_t nheads, int64_t ngroups, int64_t nchunks, int64_t nslices, int64_t hps,
                    int64_t Xsb, int64_t Xsl, int64_t Xsh) {
     constexpr int LD = lds_ld<T>(kQ);
@@ -156,9 +155,6 @@ chunk_state_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* sX = reinterpret_cast<T*>(smem_raw);        // [P][LD]   x^T scaled
     T* sM = sX + P * LD;                           // [N][LD]   B^T or C^T
-    constexpr bool PACK = sizeof(LT) == 2;         // 16-bit output: through a wave-private tile to 16-byte row stores
-    constexpr int LDO = N / 2 + 8;
-    LT* sO = reinterpret_cast<LT*>(sM + N * LD);   // PACK: [4 waves][P / 2][LDO]
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int64_t c = blockIdx.x, b = blockIdx.z;
     const int64_t g = blockIdx.y / nslices, slice = blockIdx.y % nslices;
@@ -201,38 +197,17 @@ chunk_state_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
         floatx16 acc[BM][BN];
         acc_zero(acc);
         wave_mma<BM, BN>(acc, sX + wm * (P / 2) * LD, LD, sM + wn * (N / 2) * LD, LD, 0, kQ);
-        LT* op = out + ((b * nchunks + c) * nheads + h) * (int64_t)(P * N);
-        if (PACK) {
-            LT* sOw = sO + wave * (P / 2) * LDO;
+        float* op = out + ((b * nchunks + c) * nheads + h) * (int64_t)(P * N);
 #pragma unroll
-            for (int i = 0; i < BM; ++i)
+        for (int i = 0; i < BM; ++i)
 #pragma unroll
-                for (int j = 0; j < BN; ++j)
+            for (int j = 0; j < BN; ++j)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v)
-                        sOw[(i * 32 + acc_row(lane, v)) * LDO + j * 32 + acc_col(lane)] = from_f32<LT>(acc[i][j][v]);
-            wave_lds_sync();
-            constexpr int LPR = (N / 2) / 8;           // lanes per row of this wave's [P/2][N/2] block (8 elements each)
-            constexpr int RPP = 64 / LPR;
-#pragma unroll
-            for (int ps = 0; ps < (P / 2) / RPP; ++ps) {
-                const int rl = ps * RPP + lane / LPR, cv = lane % LPR;
-                *reinterpret_cast<uint4*>(op + (wm * (P / 2) + rl) * N + wn * (N / 2) + cv * 8) =
-                    *reinterpret_cast<const uint4*>(sOw + rl * LDO + cv * 8);
-            }
-            wave_lds_sync();
-        } else {
-#pragma unroll
-            for (int i = 0; i < BM; ++i)
-#pragma unroll
-                for (int j = 0; j < BN; ++j)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int row = wm * (P / 2) + i * 32 + acc_row(lane, v);
-                        const int col = wn * (N / 2) + j * 32 + acc_col(lane);
-                        op[row * N + col] = from_f32<LT>(acc[i][j][v]);
-                    }
-        }
+                for (int v = 0; v < 16; ++v) {
+                    const int row = wm * (P / 2) + i * 32 + acc_row(lane, v);
+                    const int col = wn * (N / 2) + j * 32 + acc_col(lane);
+                    op[row * N + col] = acc[i][j][v];
+                }
     }
 }
 
@@ -256,9 +231,9 @@ chunk_state_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
 constexpr int kScanSplit = 4;
 constexpr int kDlamParts = 8;     // partial sums of dlam per (batch, head, chunk): every producer fills all of them
 
-template <typename T, int PN, bool REVERSE, typename LT>
+template <typename T, int PN, bool REVERSE>
 __global__ void __launch_bounds__(256)
-state_scan_kernel(const LT* __restrict__ local, const float* __restrict__ lam, const float* __restrict__ init,
+state_scan_kernel(const float* __restrict__ local, const float* __restrict__ lam, const float* __restrict__ init,
                   T* __restrict__ prev, float* __restrict__ final_out,
                   const T* __restrict__ sprev, float* __restrict__ dlam,
                   int64_t nheads, int64_t nchunks) {
@@ -286,7 +261,7 @@ state_scan_kernel(const LT* __restrict__ local, const float* __restrict__ lam, c
         for (int e = 0; e < EPT; ++e) {
             const int off = part0 + (e * 256 + tid) * 4;
             float loc[4];
-            loadv<LT, 4>(local + tile + off, loc);
+            loadv<float, 4>(local + tile + off, loc);
             // store the state entering (forward) / the gradient leaving (reverse) this chunk
             T o[4];
 #pragma unroll
