@@ -285,7 +285,7 @@ __device__ __forceinline__ void wave_chunk_cumsum(const void* __restrict__ dt, i
     wave_cumsum_from(A, d0, d1, l0, l1);
 }
 
-// Per (batch, head, chunk) the cumulative log-decay and dt are computed once (ld_table_kernel) into a table of
+// Per (batch, head, chunk) the cumulative log-decay and dt are computed once (ld_table_body, prep_kernel) into a table of
 // 2 * kQ floats, [ l[0..kQ) | dt[0..kQ) ], tokens past the end of the sequence holding dt = 0 and the last l.
 // Lane holds tokens `lane` and `lane + 64`.
 __device__ __forceinline__ void wave_ld_load(const float* __restrict__ ldtab, int64_t bhc, float& l0, float& l1, float& d0, float& d1) {

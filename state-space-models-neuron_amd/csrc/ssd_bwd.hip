@@ -19,18 +19,23 @@
 // Row sums and column sums are taken from the SAME fp32 tile dG^h o G, so pairs (i, j) that both lie
 // in a suffix cancel exactly and only pairs straddling the position contribute, as in exact
 // arithmetic.  (Forming dl from dy . (y - D x) with the stored bf16 y loses everything to
-// cancellation once D x dominates y.)  <dS, S_new> is exact per chunk, so rounding does not
-// accumulate along the sequence as it would with a global reverse cumulative sum (:459-461).
+// cancellation once D x dominates y.)  The state term is evaluated in the equivalent form
+//   <dS, S_new> - sum_{i>=j} (B_i . dBoff_i^h)  =  e^{Lam} <dS, S_prev> + sum_{i<j} (B_i . dBoff_i^h)
+// (a prefix instead of a suffix of the per-token terms), which avoids subtracting two large numbers that were
+// rounded differently.  Everything is exact per chunk, so rounding does not accumulate along the sequence as it
+// would with a global reverse cumulative sum (:459-461).
 //
-// Launch sequence:
-//   cb_kernel, chunk_state_kernel, state_scan_kernel          recompute G, S_prev, final state
-//   chunk_state_kernel<DSTATE>                                local dS contributions  e^{l} dy^T C
-//   state_scan_kernel<REVERSE>                                dS per chunk, <dS, S_new>, d initial state
-//   dg_kernel              per (b, chunk, group, head slice)  partial dG (heads reduced in registers), dl_diag per head
-//   off_kernel<C>, <B>     per (b, chunk, group, head slice)  partial state parts of dC / dB, dl_c per head
-//   diag_off_kernel<bwd>   per (b, chunk, group, head slice)  dx, ddt, partial dA, dD (dl assembled here)
-//   bc_final_kernel        per (b, chunk, group)              dC = dG B + dCoff, dB = dG^T C + dBoff
-//   ad_reduce_kernel                                          dA, dD (fixed order, no atomics)
+// Launch sequence (16-bit operands; fp32 operands take the kernels named in brackets):
+//   prep_kernel, state_pass16_kernel [chunk_state + state_scan]   recompute G, tables, S_prev (skipped if the caller kept them)
+//   state_pass16_kernel<REVERSE> [chunk_state<DSTATE> + state_scan<REVERSE>]
+//                                                              dS per chunk, e^{Lam} <dS, S_prev>, d initial state
+//   dg16_kernel [dg_kernel]   per (b, chunk, group, head slice)  partial dG (heads reduced in registers), dl_diag per head
+//   ssd_bwd16_kernel [off_kernel<C>, <B>, diag_off_kernel<bwd>]
+//                             per (b, chunk, group, head slice)  dx, per-token decay-gradient terms, dD partials,
+//                                                                partial state parts of dB / dC
+//   tail1_kernel              da_body: ddt, dA partials per (b, head, chunk);  slice_sum_body: partials over the head slices
+//   tail2_kernel              bc_final_body per (b, chunk, group): dC = dG B + dCoff, dB = dG^T C + dBoff;
+//                             ad_reduce_body per head: dA, dD (fixed order, no atomics)
 #include "ssd_host.hpp"
 
 namespace m2 {
@@ -310,9 +315,8 @@ off_kernel(const T* __restrict__ Arow, int64_t Asb, int64_t Asl, int64_t Ash,   
 // `tile` floats per (group, slice) tile; segment k covers threads [first_k, first_{k+1}).
 struct SliceSumSeg { const float* part; float* out; int64_t nslices, tile, first; };
 struct SliceSumArgs { SliceSumSeg seg[3]; int nseg; int64_t total; };
-__global__ void __launch_bounds__(256)
-slice_sum_kernel(const SliceSumArgs a) {
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+__device__ __forceinline__ void slice_sum_body(const SliceSumArgs& a, int64_t blk) {
+    const int64_t idx = blk * 256 + threadIdx.x;
     if (idx >= a.total) return;
     int k = 0;
     if (a.nseg > 1 && idx >= a.seg[1].first) k = 1;
@@ -323,6 +327,16 @@ slice_sum_kernel(const SliceSumArgs a) {
     floatx4 s = {0.f, 0.f, 0.f, 0.f};
     for (int64_t sl = 0; sl < sg.nslices; ++sl) s += *reinterpret_cast<const floatx4*>(sg.part + (grp * sg.nslices + sl) * sg.tile + e);
     *reinterpret_cast<floatx4*>(sg.out + grp * sg.tile + e) = s;
+}
+__global__ void __launch_bounds__(256)
+slice_sum_kernel(const SliceSumArgs a) { slice_sum_body(a, blockIdx.x); }
+// The slice sums and the per-chunk decay-gradient scan (da_body) in one launch: they are independent, and both are short.
+template <typename T>
+__global__ void __launch_bounds__(256)
+tail1_kernel(const DaArgs d, const int64_t n_da, const SliceSumArgs a) {
+    const int64_t blk = blockIdx.x;
+    if (blk < n_da) da_body<T>(d, blk);
+    else slice_sum_body(a, blk - n_da);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -345,11 +359,11 @@ __device__ __forceinline__ void wave_mma_mt(floatx16 (&acc)[1][NB], const T* __r
 }
 
 template <typename T, int N>
-__global__ void __launch_bounds__(512)
-bc_final_kernel(const float* __restrict__ dGp, const float* __restrict__ dCp, const float* __restrict__ dBp,
-                const T* __restrict__ Bt, const T* __restrict__ Ct, T* __restrict__ dB, T* __restrict__ dC,
-                int64_t seqlen, int64_t ngroups, int64_t nchunks,
-                int64_t dBsb, int64_t dBsl, int64_t dBsg, int64_t dCsb, int64_t dCsl, int64_t dCsg) {
+__device__ __forceinline__ void
+bc_final_body(const float* __restrict__ dGp, const float* __restrict__ dCp, const float* __restrict__ dBp,
+              const T* __restrict__ Bt, const T* __restrict__ Ct, T* __restrict__ dB, T* __restrict__ dC,
+              int64_t seqlen, int64_t ngroups, int64_t nchunks,
+              int64_t dBsb, int64_t dBsl, int64_t dBsg, int64_t dCsb, int64_t dCsl, int64_t dCsg, int64_t c, int64_t g, int64_t b) {
     constexpr int LDQ = lds_ld<T>(kQ);
     constexpr int NB = N / 64;
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -357,7 +371,6 @@ bc_final_kernel(const float* __restrict__ dGp, const float* __restrict__ dCp, co
     T* sT2 = sA2 + kQ * LDQ;                       // [N][LDQ]   Bt or Ct
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 31;
-    const int64_t c = blockIdx.x, g = blockIdx.y, b = blockIdx.z;
     const int64_t t0 = c * kQ;
     const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
     const int rb = wave >> 1, cb0 = (wave & 1) * 2, nb0 = (wave & 1) * NB;
@@ -441,14 +454,12 @@ bc_final_kernel(const float* __restrict__ dGp, const float* __restrict__ dCp, co
         }
 }
 
-// dA[h] = sum_{b,c} dAp[b][h][c], dD likewise.  One block per head.
-__global__ void __launch_bounds__(256)
-ad_reduce_kernel(const float* __restrict__ dAp, const float* __restrict__ dDp, float* __restrict__ dA, float* __restrict__ dD,
-                 int64_t nb, int64_t nheads, int64_t nchunks) {
-    __shared__ float red[2][4];
-    const int64_t h = blockIdx.x;
+// dA[h] = sum_{b,c} dAp[b][h][c], dD likewise (fixed order, no atomics).  One workgroup of 512 threads per head.
+__device__ __forceinline__ void ad_reduce_body(const float* __restrict__ dAp, const float* __restrict__ dDp, float* __restrict__ dA,
+                                               float* __restrict__ dD, int64_t nb, int64_t nheads, int64_t nchunks, int64_t h) {
+    __shared__ float red[2][8];
     float sa = 0.f, sd = 0.f;
-    for (int64_t e = threadIdx.x; e < nb * nchunks; e += 256) {
+    for (int64_t e = threadIdx.x; e < nb * nchunks; e += 512) {
         const int64_t b = e / nchunks, c = e % nchunks;
         sa += dAp[(b * nheads + h) * nchunks + c];
         sd += dDp[(b * nheads + h) * nchunks + c];
@@ -458,8 +469,32 @@ ad_reduce_kernel(const float* __restrict__ dAp, const float* __restrict__ dDp, f
     if (lane == 0) { red[0][wave] = sa; red[1][wave] = sd; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        dA[h] = red[0][0] + red[0][1] + red[0][2] + red[0][3];
-        if (dD) dD[h] = red[1][0] + red[1][1] + red[1][2] + red[1][3];
+        float ta = 0.f, td = 0.f;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) { ta += red[0][q]; td += red[1][q]; }
+        dA[h] = ta;
+        if (dD) dD[h] = td;
+    }
+}
+
+// The group-level finish and the per-head reductions in one launch: the first n_bc workgroups run bc_final_body for
+// (chunk, group, batch) = the index split in that order, the others ad_reduce_body for one head each.
+struct Tail2Args {
+    const float* dGp; const float* dCp; const float* dBp; const void* Bt; const void* Ct; void* dB; void* dC;
+    int64_t dBsb, dBsl, dBsg, dCsb, dCsl, dCsg;
+    const float* dAp; const float* dDp; float* dA; float* dD;
+    int64_t seqlen, ngroups, nchunks, batch, nheads, n_bc;
+};
+template <typename T, int N>
+__global__ void __launch_bounds__(512)
+tail2_kernel(const Tail2Args a) {
+    const int64_t blk = blockIdx.x;
+    if (blk < a.n_bc) {
+        const int64_t c = blk % a.nchunks, g = (blk / a.nchunks) % a.ngroups, b = blk / (a.nchunks * a.ngroups);
+        bc_final_body<T, N>(a.dGp, a.dCp, a.dBp, static_cast<const T*>(a.Bt), static_cast<const T*>(a.Ct), static_cast<T*>(a.dB),
+                            static_cast<T*>(a.dC), a.seqlen, a.ngroups, a.nchunks, a.dBsb, a.dBsl, a.dBsg, a.dCsb, a.dCsl, a.dCsg, c, g, b);
+    } else {
+        ad_reduce_body(a.dAp, a.dDp, a.dA, a.dD, a.batch, a.nheads, a.nchunks, blk - a.n_bc);
     }
 }
 
@@ -542,6 +577,8 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         }
         if ((rc = check_launch("ssd dg_kernel"))) return rc;
     }
+    DaArgs da{};
+    bool have_da = false;
     {
         if constexpr (!bwd16_ok<T, P, N>()) {
         auto kc = off_kernel<T, P, N, true>;
@@ -591,10 +628,12 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
             if ((rc = allow_smem(k, sm))) return rc;
             k<<<grid_b, 512, sm, st>>>(m);
             if ((rc = check_launch("ssd_bwd16_kernel"))) return rc;
-            da_kernel<T><<<(unsigned)ceil_div(p->batch * p->nheads * nc, (int64_t)4), 256, 0, st>>>(
-                w.ldtab, p->A, w.dl, w.dlc, w.dlam, w.dirp, w.rbp, w.dDp8,
-                p->ddt, dt_f32, p->ddt_stride_b, p->ddt_stride_l, w.dAp, w.dDp, p->seqlen, p->nheads, nc, p->batch * p->nheads * nc);
-            if ((rc = check_launch("ssd da_kernel"))) return rc;
+            // the per-chunk scan that turns these per-token terms into ddt and dA partials runs with the slice sums below
+            have_da = true;
+            da.ldtab = w.ldtab; da.A = p->A; da.dl_diag = w.dl; da.dl_c = w.dlc; da.dlam = w.dlam;
+            da.dirp = w.dirp; da.rbp = w.rbp; da.dDp8 = w.dDp8;
+            da.ddt = p->ddt; da.dt_f32 = dt_f32; da.ddt_sb = p->ddt_stride_b; da.ddt_sl = p->ddt_stride_l; da.dAp = w.dAp; da.dDp = w.dDp;
+            da.seqlen = p->seqlen; da.nheads = p->nheads; da.nchunks = nc; da.total = p->batch * p->nheads * nc;
         } else {
             auto k = diag_off_kernel<T, P, N, true>;
             const size_t sm = diag_smem<T, P, N, true>();
@@ -604,9 +643,6 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         if ((rc = check_launch("ssd diag_off_kernel<bwd>"))) return rc;
     }
     {
-        auto k = bc_final_kernel<T, N>;
-        const size_t sm = bcf_smem<T, N>();
-        if ((rc = allow_smem(k, sm))) return rc;
         const int64_t ngrp = p->batch * nc * p->ngroups;
         const float *gs = w.dGp, *cs = w.dCp, *bs = w.dBp;
         {
@@ -622,16 +658,22 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
             add(w.dCp, w.dCs, w.ns_c, (int64_t)kQ * N, &cs);
             add(w.dBp, w.dBs, w.ns_b, (int64_t)kQ * N, &bs);
             sa.total = first;
-            if (sa.nseg > 0) slice_sum_kernel<<<(unsigned)ceil_div(first, (int64_t)256), 256, 0, st>>>(sa);
+            const int64_t n_ss = ceil_div(first, (int64_t)256), n_da = have_da ? ceil_div(da.total, (int64_t)4) : 0;
+            if (have_da) tail1_kernel<T><<<(unsigned)(n_da + n_ss), 256, 0, st>>>(da, n_da, sa);
+            else if (n_ss > 0) slice_sum_kernel<<<(unsigned)n_ss, 256, 0, st>>>(sa);
         }
-        if ((rc = check_launch("ssd slice_sum_kernel"))) return rc;
-        k<<<dim3((unsigned)nc, (unsigned)p->ngroups, (unsigned)p->batch), 512, sm, st>>>(
-            gs, cs, bs, static_cast<const T*>(w.Bt), static_cast<const T*>(w.Ct),
-            static_cast<T*>(p->dB), static_cast<T*>(p->dC), p->seqlen, p->ngroups, nc,
-            p->dB_stride_b, p->dB_stride_l, p->dB_stride_g, p->dC_stride_b, p->dC_stride_l, p->dC_stride_g);
-        if ((rc = check_launch("ssd bc_final_kernel"))) return rc;
-        ad_reduce_kernel<<<(unsigned)p->nheads, 256, 0, st>>>(w.dAp, w.dDp, p->dA, p->D ? p->dD : nullptr, p->batch, p->nheads, nc);
-        if ((rc = check_launch("ssd ad_reduce_kernel"))) return rc;
+        if ((rc = check_launch("ssd tail1_kernel"))) return rc;
+        auto k = tail2_kernel<T, N>;
+        const size_t sm = bcf_smem<T, N>();
+        if ((rc = allow_smem(k, sm))) return rc;
+        Tail2Args ta;
+        ta.dGp = gs; ta.dCp = cs; ta.dBp = bs; ta.Bt = w.Bt; ta.Ct = w.Ct; ta.dB = p->dB; ta.dC = p->dC;
+        ta.dBsb = p->dB_stride_b; ta.dBsl = p->dB_stride_l; ta.dBsg = p->dB_stride_g;
+        ta.dCsb = p->dC_stride_b; ta.dCsl = p->dC_stride_l; ta.dCsg = p->dC_stride_g;
+        ta.dAp = w.dAp; ta.dDp = w.dDp; ta.dA = p->dA; ta.dD = p->D ? p->dD : nullptr;
+        ta.seqlen = p->seqlen; ta.ngroups = p->ngroups; ta.nchunks = nc; ta.batch = p->batch; ta.nheads = p->nheads; ta.n_bc = ngrp;
+        k<<<(unsigned)(ngrp + p->nheads), 512, sm, st>>>(ta);
+        if ((rc = check_launch("ssd tail2_kernel"))) return rc;
     }
     return M2_OK;
 }

@@ -17,7 +17,7 @@
 //            accumulated over the workgroup's heads in registers (row scale applied in fp32 after the MFMA, so both
 //            operands are exact copies of the inputs) and written once at the end.
 // The decay is factorised per row block around its LAST token (see ssd_diag.hpp), with the exact per-element
-// fallback when the block's range exceeds kMaxRange.  ddt and dA need a scan over the chunk and are left to da_kernel.
+// fallback when the block's range exceeds kMaxRange.  ddt and dA need a scan over the chunk and are left to da_body (tail1_kernel).
 #pragma once
 #include "ssd_y.hpp"
 
@@ -402,17 +402,24 @@ ssd_bwd16_kernel(const Bwd16Args a) {
 
 // Per (batch, head, chunk): da_t = sum_{i>=t} (dl_diag_i + dl_c_i) + sum_{j<t} rb_j + dlam,  ddt_t = A da_t + dir_t,
 // dA partial = sum_t da_t dt_t, dD partial = sum of the per-wave partials.  One wave per (b, h, c), four per
-// workgroup; lanes hold the tokens in reverse order (127 - lane, 63 - lane), so the suffix over tokens is an inclusive
+// workgroup (the first four waves of workgroup `blk` of tail1_kernel); lanes hold the tokens in reverse order (127 - lane, 63 - lane), so the suffix over tokens is an inclusive
 // prefix over lanes and the exclusive prefix over tokens an exclusive suffix over lanes.
+struct DaArgs {
+    const float* ldtab; const float* A; const float* dl_diag; const float* dl_c; const float* dlam;
+    const float* dirp; const float* rbp; const float* dDp8;
+    void* ddt; int dt_f32; int64_t ddt_sb, ddt_sl; float* dAp; float* dDp;
+    int64_t seqlen, nheads, nchunks, total;
+};
 template <typename T>
-__global__ void __launch_bounds__(256)
-da_kernel(const float* __restrict__ ldtab, const float* __restrict__ A,
-          const float* __restrict__ dl_diag, const float* __restrict__ dl_c, const float* __restrict__ dlam,
-          const float* __restrict__ dirp, const float* __restrict__ rbp, const float* __restrict__ dDp8,
-          void* __restrict__ ddt, int dt_f32, int64_t ddt_sb, int64_t ddt_sl, float* __restrict__ dAp, float* __restrict__ dDp,
-          int64_t seqlen, int64_t nheads, int64_t nchunks, int64_t total) {
+__device__ __forceinline__ void da_body(const DaArgs& q, int64_t blk) {
+    const float* __restrict__ ldtab = q.ldtab; const float* __restrict__ A = q.A;
+    const float* __restrict__ dl_diag = q.dl_diag; const float* __restrict__ dl_c = q.dl_c; const float* __restrict__ dlam = q.dlam;
+    const float* __restrict__ dirp = q.dirp; const float* __restrict__ rbp = q.rbp; const float* __restrict__ dDp8 = q.dDp8;
+    void* __restrict__ ddt = q.ddt; const int dt_f32 = q.dt_f32; const int64_t ddt_sb = q.ddt_sb, ddt_sl = q.ddt_sl;
+    float* __restrict__ dAp = q.dAp; float* __restrict__ dDp = q.dDp;
+    const int64_t seqlen = q.seqlen, nheads = q.nheads, nchunks = q.nchunks, total = q.total;
     const int lane = threadIdx.x & 63;
-    const int64_t bhc = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t bhc = blk * 4 + (threadIdx.x >> 6);
     if (bhc >= total) return;
     const int64_t c = bhc % nchunks, h = (bhc / nchunks) % nheads, b = bhc / (nchunks * nheads);
     const int64_t t0 = c * kQ;

@@ -1,15 +1,15 @@
 // SSD chunked-scan forward for gfx950.
 //
 // Replaces the reference's NKI kernel mamba_kernel_ (mamba2/mamba2_kernel.py:67-170), which walks
-// the chunks of one (batch, head) sequentially with the state on chip.  Here the work is split so
-// that every (batch, head, chunk) tile is an independent workgroup (thousands of them for 256 CUs)
-// and only a cheap elementwise recurrence is sequential in the chunk index:
+// the chunks of one (batch, head) sequentially with the state on chip.  Here only the state recurrence
+// is sequential in the chunk index; everything else is one independent workgroup per (batch, chunk,
+// group) that loops over a slice of the group's heads:
 //
-//   0. ld_table_kernel     l = cumsum(A dt) per chunk        per (b, head, chunk)    scan
-//   1. cb_kernel           G = C B^T                         per (b, chunk, group)   MFMA
-//   2. chunk_state_kernel  local state B^T (decay o dt o X)  per (b, chunk, head)    MFMA
-//   3. state_scan_kernel   S_prev(c), final state            per (b, head)           fp32 FMA
-//   4. ssd_y16_kernel (16-bit) / diag_off_kernel<false>      Y = (L o G)(dt o X) + e^l C S_prev + D X   MFMA
+//   1. prep_kernel         l = cumsum(A dt) per (b, head, chunk);  G = C B^T (+ operand tiles) per (b, chunk, group)
+//   2. states entering the chunks, final state
+//        16-bit: state_pass16_kernel   contributions B^T (decay o dt o X) and recurrence fused, per (b, head)
+//        fp32  : chunk_state_kernel + state_scan_kernel
+//   3. ssd_y16_kernel (16-bit) / diag_off_kernel<false>      Y = (L o G)(dt o X) + e^l C S_prev + D X   MFMA
 //
 // Extensions over the reference kernel: optional initial state, final-state output, any batch,
 // ragged sequence length (tokens past the end behave as dt = 0 and are never written).

@@ -165,19 +165,23 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
     const int dt_f32 = p->dt_dtype == M2_F32;
     int rc;
     {
-        const int64_t total = p->batch * p->nheads * nc;
-        ld_table_kernel<T><<<(unsigned)ceil_div(total, (int64_t)4), 256, 0, st>>>(p->dt, dt_f32, p->A, w.ldtab, w.lam, p->seqlen, p->nheads, nc, total,
-                                                                                p->dt_stride_b, p->dt_stride_l);
-        if ((rc = check_launch("ssd ld_table_kernel"))) return rc;
-    }
-    {
-        auto k = cb_kernel<T, N>;
+        // decay tables and G = C B^T (+ operand tiles), one launch
+        auto k = prep_kernel<T, N>;
         const size_t sm = cb_smem<T>();
         if ((rc = allow_smem(k, sm))) return rc;
-        k<<<dim3((unsigned)nc, (unsigned)p->ngroups, (unsigned)p->batch), 256, sm, st>>>(
-            Bm, Cm, w.G, static_cast<T*>(w.Gm), static_cast<T*>(w.Gmt), static_cast<T*>(w.Bt), static_cast<T*>(w.Ct), p->seqlen, p->ngroups, nc, p->B_stride_b, p->B_stride_l, p->B_stride_g,
-            p->C_stride_b, p->C_stride_l, p->C_stride_g);
-        if ((rc = check_launch("ssd cb_kernel"))) return rc;
+        PrepArgs pa;
+        pa.Bm = Bm; pa.Cm = Cm; pa.Gf = w.G; pa.Gm = w.Gm; pa.Gmt = w.Gmt; pa.Bt = w.Bt; pa.Ct = w.Ct;
+        pa.Bsb = p->B_stride_b; pa.Bsl = p->B_stride_l; pa.Bsg = p->B_stride_g;
+        pa.Csb = p->C_stride_b; pa.Csl = p->C_stride_l; pa.Csg = p->C_stride_g;
+        pa.dt = p->dt; pa.dt_f32 = dt_f32; pa.A = p->A; pa.ldtab = w.ldtab; pa.lam = w.lam;
+        pa.dtsb = p->dt_stride_b; pa.dtsl = p->dt_stride_l;
+        pa.seqlen = p->seqlen; pa.nheads = p->nheads; pa.ngroups = p->ngroups; pa.nchunks = nc;
+        pa.total_bhc = p->batch * p->nheads * nc;
+        pa.n_cb = nc * p->ngroups * p->batch;
+        const int64_t blocks = pa.n_cb + ceil_div(pa.total_bhc, (int64_t)4);
+        M2_REQUIRE(blocks < ((int64_t)1 << 31), M2_ERR_SHAPE, "ssd: too many workgroups");
+        k<<<(unsigned)blocks, 256, sm, st>>>(pa);
+        if ((rc = check_launch("ssd prep_kernel"))) return rc;
     }
     if constexpr (sizeof(T) == 2) {
         // 16-bit operands: contributions and recurrence in one pass, running state in registers

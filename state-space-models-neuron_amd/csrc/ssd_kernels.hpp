@@ -32,7 +32,7 @@ namespace m2 {
 //   Gmt [kQ][kQ] T               its transpose: Gmt[j][i] = G[i][j] for i >= j (backward dx term, rows j)
 //   Bt, Ct N x kQ T              B and C transposed (tokens contiguous), laid out by mt_offset: MFMA operands of the
 //                                chunk-state products
-// grid (nchunks, ngroups, batch), 256 threads.  The upper-right 64x64 quadrant of G is never consumed and is
+// One workgroup of 256 threads per (chunk, group, batch).  The upper-right 64x64 quadrant of G is never consumed and is
 // neither computed nor written.
 // Element offset of the 8 tokens s0 .. s0 + 7 (s0 a multiple of 8) of state column n inside a transposed B / C tile.
 //   fp32   : [N][kQ], tokens contiguous (rows staged into LDS by chunk_state_kernel);
@@ -46,11 +46,11 @@ __device__ __forceinline__ int64_t mt_offset(int n, int s0) {
 }
 
 template <typename T, int N>
-__global__ void __launch_bounds__(256)
-cb_kernel(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict__ Gf, T* __restrict__ Gm, T* __restrict__ Gmt,
-          T* __restrict__ Bt, T* __restrict__ Ct,
-          int64_t seqlen, int64_t ngroups, int64_t nchunks,
-          int64_t Bsb, int64_t Bsl, int64_t Bsg, int64_t Csb, int64_t Csl, int64_t Csg) {
+__device__ __forceinline__ void
+cb_body(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict__ Gf, T* __restrict__ Gm, T* __restrict__ Gmt,
+        T* __restrict__ Bt, T* __restrict__ Ct,
+        int64_t seqlen, int64_t ngroups, int64_t nchunks,
+        int64_t Bsb, int64_t Bsl, int64_t Bsg, int64_t Csb, int64_t Csl, int64_t Csg, int64_t c, int64_t g, int64_t b) {
     constexpr int KB = 64;
     constexpr int LD = lds_ld<T>(KB);
     constexpr int V = VecTraits<T>::kVec;
@@ -58,7 +58,6 @@ cb_kernel(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict_
     T* sC = reinterpret_cast<T*>(smem_raw);
     T* sB = sC + kQ * LD;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int64_t c = blockIdx.x, g = blockIdx.y, b = blockIdx.z;
     const int64_t t0 = c * kQ;
     const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
     const T* Bp = Bm + b * Bsb + t0 * Bsl + g * Bsg;
@@ -114,16 +113,16 @@ cb_kernel(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict_
 }
 
 // ------------------------------------------------------------------------------------------
-// Cumulative log-decay table: one wave per (batch, head, chunk); ldtab[bhc] = [ l[0..kQ) | dt[0..kQ) ] in fp32,
+// Cumulative log-decay table: one wave per (batch, head, chunk), four per workgroup; ldtab[bhc] = [ l[0..kQ) | dt[0..kQ) ] in fp32,
 // l = inclusive cumsum of A_h dt within the chunk, lam[bhc] = l[kQ-1].  Every other kernel reads this table instead
 // of gathering dt (stride = nheads elements) and scanning it again per head.
 template <typename T>
-__global__ void __launch_bounds__(256)
-ld_table_kernel(const void* __restrict__ dt, int dt_f32, const float* __restrict__ A, float* __restrict__ ldtab,
-                float* __restrict__ lam, int64_t seqlen, int64_t nheads, int64_t nchunks, int64_t total,
-                int64_t dtsb, int64_t dtsl) {
+__device__ __forceinline__ void
+ld_table_body(const void* __restrict__ dt, int dt_f32, const float* __restrict__ A, float* __restrict__ ldtab,
+              float* __restrict__ lam, int64_t seqlen, int64_t nheads, int64_t nchunks, int64_t total,
+              int64_t dtsb, int64_t dtsl, int64_t blk) {
     const int lane = threadIdx.x & 63;
-    const int64_t bhc = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t bhc = blk * 4 + (threadIdx.x >> 6);
     if (bhc >= total) return;
     const int64_t c = bhc % nchunks, h = (bhc / nchunks) % nheads, b = bhc / (nchunks * nheads);
     const int64_t t0 = c * kQ;
@@ -135,12 +134,34 @@ ld_table_kernel(const void* __restrict__ dt, int dt_f32, const float* __restrict
     if (lane == 63) lam[bhc] = l1;
 }
 
+// Both preparations in one launch (they are independent, and either alone leaves most of the GPU idle): the first
+// n_cb workgroups run cb_body for (chunk, group, batch) = the index split in that order, the others ld_table_body.
+struct PrepArgs {
+    const void* Bm; const void* Cm; float* Gf; void* Gm; void* Gmt; void* Bt; void* Ct;
+    int64_t Bsb, Bsl, Bsg, Csb, Csl, Csg;
+    const void* dt; int dt_f32; const float* A; float* ldtab; float* lam; int64_t dtsb, dtsl;
+    int64_t seqlen, nheads, ngroups, nchunks, total_bhc, n_cb;
+};
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+prep_kernel(const PrepArgs a) {
+    const int64_t blk = blockIdx.x;
+    if (blk < a.n_cb) {
+        const int64_t c = blk % a.nchunks, g = (blk / a.nchunks) % a.ngroups, b = blk / (a.nchunks * a.ngroups);
+        cb_body<T, N>(static_cast<const T*>(a.Bm), static_cast<const T*>(a.Cm), a.Gf, static_cast<T*>(a.Gm), static_cast<T*>(a.Gmt),
+                      static_cast<T*>(a.Bt), static_cast<T*>(a.Ct), a.seqlen, a.ngroups, a.nchunks,
+                      a.Bsb, a.Bsl, a.Bsg, a.Csb, a.Csl, a.Csg, c, g, b);
+    } else {
+        ld_table_body<T>(a.dt, a.dt_f32, a.A, a.ldtab, a.lam, a.seqlen, a.nheads, a.nchunks, a.total_bhc, a.dtsb, a.dtsl, blk - a.n_cb);
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // Local chunk state.  grid (nchunks, ngroups * nslices, batch), 256 threads; a workgroup loops over `hps` heads.
 //   DSTATE == false:  out[p][n] = sum_j (dt_j e^{Lam-l_j}) x[j][p] * B[j][n]      (forward)
 //   DSTATE == true :  out[p][n] = sum_i e^{l_i} dy[i][p] * C[i][n]                (backward)
 // Used for fp32 operands (16-bit operands take state_pass16_kernel, which fuses this with the recurrence); `out` is fp32.
-// `X` is x or dy; `Mt` is the group's B or C tile already transposed to [N][kQ] (tokens contiguous) by cb_kernel,
+// `X` is x or dy; `Mt` is the group's B or C tile already transposed to [N][kQ] (tokens contiguous) by cb_body (prep_kernel),
 // staged into LDS once per workgroup.  Per head only the x tile moves: it is loaded 16 bytes at a time, scaled in
 // fp32 and written transposed; the next head's tile is prefetched into registers while the MFMAs run.
 template <typename T, int P, int N, bool DSTATE>

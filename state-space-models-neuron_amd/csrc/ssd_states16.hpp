@@ -8,7 +8,7 @@
 //
 // grid (nheads * NSPLIT, batch), 2 x NWG waves; a workgroup owns N / NSPLIT columns of the [P][N] state, wave w rows
 // [ (w & 1) P/2, +P/2 ) x one NWG-th of those columns, as 32x32 MFMA accumulator blocks.  Per chunk the MFMA computes  X_scaled^T [P x kQ] * M [kQ x N]:
-//   * M (B or C of the group) comes from the transposed tiles that cb_kernel wrote in MFMA operand order: a wave's
+//   * M (B or C of the group) comes from the transposed tiles that prep_kernel wrote in MFMA operand order: a wave's
 //     B-operand fragment is one contiguous KiB of global memory, loaded straight into registers at the top of the
 //     chunk's iteration (the tile is shared by all heads of the group and stays in L2);
 //   * x / dy rows are loaded one chunk ahead into registers, scaled per token in fp32, rounded once and written
