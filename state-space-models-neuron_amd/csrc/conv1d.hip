@@ -338,16 +338,26 @@ __global__ void conv_zero_kernel(uint16_t* __restrict__ p, int64_t n) {
     if (i < n) p[i] = 0;
 }
 
-// Second stage: sum the per-block partials.  One thread per (channel, tap-or-bias).
-__global__ void conv_reduce_partials_kernel(const float* __restrict__ part, int64_t nslots, int64_t C, int k,
-                                            void* __restrict__ dw, void* __restrict__ db, int pd) {
-    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+// Second stage: sum the per-block partials.  Four adjacent lanes per (channel, tap-or-bias), each a quarter of the
+// slots (fixed order), combined by two shuffles.
+__global__ void __launch_bounds__(256)
+conv_reduce_partials_kernel(const float* __restrict__ part, int64_t nslots, int64_t C, int k,
+                            void* __restrict__ dw, void* __restrict__ db, int pd) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t e = t >> 2;
+    const int q = (int)(t & 3);
     const int kk = k + 1;
-    if (e >= C * kk) return;
-    const int64_t c = e / kk;
-    const int i = (int)(e % kk);
+    const bool live = e < C * kk;
+    const int64_t c = live ? e / kk : 0;
+    const int i = live ? (int)(e % kk) : 0;
     float s = 0.f;
-    for (int64_t r = 0; r < nslots; ++r) s += part[(r * C + c) * kk + i];
+    if (live) {
+#pragma unroll 4
+        for (int64_t r = q; r < nslots; r += 4) s += part[(r * C + c) * kk + i];
+    }
+    s += __shfl_xor(s, 1, 64);
+    s += __shfl_xor(s, 2, 64);
+    if (!live || q != 0) return;
     if (i < k) st_param(dw, pd, c * k + i, s);
     else if (db) st_param(db, pd, c, s);
 }
@@ -532,7 +542,7 @@ int launch_bwd(const m2_conv1d_params* p, hipStream_t st) {
         }
         int rc = check_launch("conv1d_bwd");
         if (rc) return rc;
-        conv_reduce_partials_kernel<<<(unsigned)ceil_div(C * 5, 256), 256, 0, st>>>(part, nslots, C, 4, p->dw, p->db, p->param_dtype);
+        conv_reduce_partials_kernel<<<(unsigned)ceil_div(C * 5 * 4, (int64_t)256), 256, 0, st>>>(part, nslots, C, 4, p->dw, p->db, p->param_dtype);
         return check_launch("conv1d_bwd_reduce");
     }
     const int64_t total = nb * l * C;

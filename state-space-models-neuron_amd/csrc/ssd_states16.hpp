@@ -20,17 +20,6 @@
 
 namespace m2 {
 
-// the two 16-bit elements of a 32-bit word as fp32, and back (round to nearest even)
-template <typename T> __device__ __forceinline__ float unpack_lo(uint32_t w);
-template <typename T> __device__ __forceinline__ float unpack_hi(uint32_t w);
-template <> __device__ __forceinline__ float unpack_lo<bf16_t>(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
-template <> __device__ __forceinline__ float unpack_hi<bf16_t>(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
-template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    typedef T tvec2 __attribute__((ext_vector_type(2)));
-    const tvec2 v = {from_f32<T>(lo), from_f32<T>(hi)};
-    return __builtin_bit_cast(uint32_t, v);
-}
-
 struct StatePassArgs {
     const void* X; int64_t X_sb, X_sl, X_sh;      // x (forward) / dy (reverse): [b][l][h][P]
     const float* ldtab;                            // [b][h][c][ l kQ | dt kQ ]
