@@ -28,7 +28,7 @@ template <int N> constexpr int bwd16_clds() { return N / 16 > 4 ? N / 32 : 0; }
 template <int P, int N>
 constexpr size_t bwd16_smem() {
     return (size_t)2 * ((2 * P * N + 2 * kQ * P) * 2 + 2 * kQ * sizeof(float)) + (size_t)4 * (kQ + 32) * sizeof(float) + (size_t)4 * 8 * P * sizeof(float) +
-           (size_t)4 * 32 * (bwd16_clds<N>() * 16 + 8) * 2;
+           (size_t)4 * 32 * (bwd16_clds<N>() * 16 + 8) * 2 + (size_t)4 * 64 * sizeof(float);
 }
 template <typename T, int P, int N>
 constexpr bool bwd16_ok() { return sizeof(T) == 2 && bwd16_smem<P, N>() <= 160 * 1024; }
@@ -66,6 +66,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
     constexpr int KCL = bwd16_clds<N>(), KCR = KSN - KCL;            // C-row fragments in LDS / in registers
     constexpr int LDC = KCL * 16 + 8;
     T* sFC = reinterpret_cast<T*>(sY + 4 * 8 * P);                   // [4 role-A waves][32][LDC]
+    float* wsB_all = reinterpret_cast<float*>(sFC + 4 * 32 * LDC);   // [4 role-B waves][ dB-side 32 | dC-side 32 ] row scales
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 31, half = lane >> 5;
@@ -203,14 +204,10 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                 }
                 float dv[16];
                 row_dot(yo, cY, dv);
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int row = row0 + acc_row(lane, v);
-                    dv[v] *= row < valid ? __expf(sl[row]) : 0.f;
-                }
                 int ri;
                 const float tot = half_wave_reduce16(dv, &ri);
-                if ((lane & 1) == 0) a.dlc[bhc * kQ + row0 + acc_row(lane, ri)] = tot;
+                const int row = row0 + acc_row(lane, ri);          // the row scale is applied to the row total
+                if ((lane & 1) == 0) a.dlc[bhc * kQ + row] = row < valid ? tot * __expf(sl[row]) : 0.f;
             }
 
             __builtin_amdgcn_sched_barrier(0);
@@ -237,12 +234,10 @@ ssd_bwd16_kernel(const Bwd16Args a) {
             {
                 float rv[16];
                 row_dot(acc, cX, rv);
-#pragma unroll
-                for (int v = 0; v < 16; ++v) rv[v] *= fin_scale(v);
                 int ri;
                 const float tot = half_wave_reduce16(rv, &ri);
                 const int row = row0 + acc_row(lane, ri);
-                if ((lane & 1) == 0) a.rbp[bhc * kQ + row] = tot * sd[row];
+                if ((lane & 1) == 0) a.rbp[bhc * kQ + row] = tot * fin_scale(ri) * sd[row];
             }
 
             __builtin_amdgcn_sched_barrier(0);
@@ -344,6 +339,14 @@ ssd_bwd16_kernel(const Bwd16Args a) {
             wait_vmem_all();
             const float* sl = sLD + buf * 2 * kQ;
             const float* sd = sl + kQ;
+            // row scales of this wave's 32 tokens, one exponential per token: dt_j e^{Lam - l_j} (dB side, lanes 0-31) and
+            // e^{l_i} (dC side, lanes 32-63; 0 past the end of the sequence)
+            float* wsw = wsB_all + rbk * 64;
+            {
+                const int row = row0 + r;
+                const float lr = sl[row];
+                wsw[lane] = half == 0 ? sd[row] * __expf(sl[kQ - 1] - lr) : (row < valid ? __expf(lr) : 0.f);
+            }
             __syncthreads();
             if (hh + 1 < a.hps) issue_tiles(h + 1, buf ^ 1);
             const T* cS = tiles + buf * TILES;
@@ -353,16 +356,13 @@ ssd_bwd16_kernel(const Bwd16Args a) {
             const int tok = row0 + r;
             // t[n-block] = sum_p Rows[tok][p] * St[p][n]: rows as they lie (A operand), the state tile through transpose reads
             auto rows_times_state = [&](const T* Rows, const T* St, bool side_b, floatx16 (&accum)[1][NBN]) {
-                // row scales of this lane's 16 accumulator rows: dt_j e^{Lam - l_j} (dB side) or e^{l_i} (dC side; 0 past the end)
+                // row scales of this lane's 16 accumulator rows (rows 8 q + 4 half + 0..3: four consecutive table entries)
                 float ws[16];
-                {
-                    const float Lam = sl[kQ - 1];
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int row = row0 + acc_row(lane, v);
-                        const float lr = sl[row];
-                        ws[v] = side_b ? sd[row] * __expf(Lam - lr) : (row < valid ? __expf(lr) : 0.f);
-                    }
+                for (int q = 0; q < 4; ++q) {
+                    const floatx4 w4 = *reinterpret_cast<const floatx4*>(wsw + (side_b ? 0 : 32) + 8 * q + 4 * half);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) ws[4 * q + e] = w4[e];
                 }
 #pragma unroll
                 for (int jn = 0; jn < NBN; ++jn) {
