@@ -287,10 +287,13 @@ ssd_bwd16_kernel(const Bwd16Args a) {
             float dD_loc = 0.f;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
+                // the final row scales of accumulator rows 8 q + 4 half + 0..3: four consecutive table entries
+                floatx4 fs = {1.f, 1.f, 1.f, 1.f};
+                if (fast) fs = *reinterpret_cast<const floatx4*>(wu + 8 * q + 4 * half);
 #pragma unroll
                 for (int j = 0; j < BN; ++j)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) sYw[(4 * half + e) * P + j * 32 + r] = acc[0][j][4 * q + e] * fin_scale(4 * q + e);
+                    for (int e = 0; e < 4; ++e) sYw[(4 * half + e) * P + j * 32 + r] = acc[0][j][4 * q + e] * fs[e];
                 wave_lds_sync();
 #pragma unroll
                 for (int ps = 0; ps < 8 / RPP; ++ps) {

@@ -131,7 +131,11 @@ dg16_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
         const float vj = __expf(fminf(l_first - lj, kMaxRange)) * dtj;
         float ui[16];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) ui[v] = sl[rb * 32 + acc_row(lane, v)];
+        for (int q = 0; q < 4; ++q) {      // accumulator rows 8 q + 4 half + 0..3: four consecutive table entries
+            const floatx4 l4 = *reinterpret_cast<const floatx4*>(sl + rb * 32 + 8 * q + 4 * half);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ui[4 * q + e] = l4[e];
+        }
         if (fast) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) ui[v] = __expf(ui[v] - l_first) * vj;      // u_i * v_j

@@ -187,7 +187,6 @@ ssd_y16_kernel(const DiagArgs a) {
 
         const float off_fast = __expf(lref);
         auto off_scale = [&](int v) -> float { return fast ? off_fast : __expf(sl[row0 + acc_row(lane, v)]); };
-        auto fin_scale = [&](int v) -> float { return fast ? wu[acc_row(lane, v)] : 1.f; };
 
         // ---- off-diagonal term: C rows (registers) x S_prev (LDS, natural layout)
         floatx16 acc[1][BN];
@@ -256,10 +255,13 @@ ssd_y16_kernel(const DiagArgs a) {
         T* Yp = static_cast<T*>(a.Y) + b * a.Y_sb + t0 * a.Y_sl + h * a.Y_sh;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
+            // the final row scales of accumulator rows 8 q + 4 half + 0..3: four consecutive table entries
+            floatx4 fs = {1.f, 1.f, 1.f, 1.f};
+            if (fast) fs = *reinterpret_cast<const floatx4*>(wu + 8 * q + 4 * half);
 #pragma unroll
             for (int j = 0; j < BN; ++j)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) sYw[(4 * half + e) * P + j * 32 + r] = acc[0][j][4 * q + e] * fin_scale(4 * q + e);
+                for (int e = 0; e < 4; ++e) sYw[(4 * half + e) * P + j * 32 + r] = acc[0][j][4 * q + e] * fs[e];
             wave_lds_sync();
 #pragma unroll
             for (int ps = 0; ps < 8 / RPP; ++ps) {
