@@ -90,6 +90,18 @@ template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float 
     return __builtin_bit_cast(uint32_t, v);
 }
 
+// Lane-pair exchange (lanes l and l + 32): lo = { own a | partner's b }, hi = { partner's a | own b } for the lower | upper
+// half of the wave (v_permlane32_swap).  With the transposed 32x32 accumulator layout (a lane and its partner hold the two
+// halves of each 8-element group of one row) this leaves every lane with whole groups of 8 consecutive elements.
+// (The scalars are passed by value on purpose: a bit cast applied directly to a vector element reads element 0.)
+__device__ __forceinline__ void pair_swap(float a, float b, float& lo, float& hi) {
+    const uint32_t ua = __builtin_bit_cast(uint32_t, a), ub = __builtin_bit_cast(uint32_t, b);
+    const auto sw = __builtin_amdgcn_permlane32_swap(ua, ub, false, false);
+    const uint32_t r0 = sw[0], r1 = sw[1];
+    lo = __builtin_bit_cast(float, r0);
+    hi = __builtin_bit_cast(float, r1);
+}
+
 // Makes a fragment opaque to the optimiser at this point (no instruction is emitted).  Used on loop-invariant
 // fragments that are re-scaled inside a loop: without it the bf16 -> fp32 unpacking of the fragment is hoisted out of
 // the loop and the fragment then occupies eight fp32 registers instead of four packed ones for the whole loop.

@@ -17,8 +17,9 @@
 // possible; bank conflicts are avoided by an XOR swizzle of the slot index inside each row instead (each lane
 // simply fetches the global piece that belongs in its slot).
 // The head-independent operands stay in registers for the whole loop: the causal C B^T fragments and the C row
-// fragments.  The epilogue goes through a small wave-private fp32 LDS tile so that y leaves in 16-byte
-// row-contiguous stores, rounded once.
+// fragments.  The MFMAs are issued with swapped operands, so a lane's accumulators belong to ONE token (transposed
+// output block): decay scales and the D x term are lane-local, and after one lane-pair swap per 4-channel group
+// (v_permlane32_swap) y leaves in 16-byte row-contiguous stores, rounded once, without a pass through LDS.
 #pragma once
 #include "ssd_diag.hpp"
 
@@ -86,7 +87,7 @@ template <int SPR> __device__ __forceinline__ int tile_swz(int row) {
 
 template <int P, int N>
 constexpr size_t y16_smem() {
-    return (size_t)2 * ((P * N + kQ * P) * 2 + 2 * kQ * sizeof(float)) + (size_t)4 * (kQ + 32) * sizeof(float) + (size_t)4 * 8 * P * sizeof(float);
+    return (size_t)2 * ((P * N + kQ * P) * 2 + 2 * kQ * sizeof(float)) + (size_t)4 * (kQ + 32) * sizeof(float);
 }
 
 template <typename T, int P, int N>
@@ -102,7 +103,6 @@ ssd_y16_kernel(const DiagArgs a) {
     T* sX = sS + 2 * P * N;                                       // [2][kQ][P]    swizzled slots
     float* sLD = reinterpret_cast<float*>(sX + 2 * kQ * P);       // [2][ l kQ | dt kQ ]
     float* wt_all = sLD + 2 * 2 * kQ;                             // [4 waves][wv kQ | wu 32]
-    float* sY = wt_all + 4 * TAB;                                 // [4 waves][8][P]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 31, half = lane >> 5;
@@ -114,7 +114,6 @@ ssd_y16_kernel(const DiagArgs a) {
     const int row0 = wave * 32;
     float* wv = wt_all + wave * TAB;
     float* wu = wv + kQ;          // [32]: rows row0 .. row0 + 31
-    float* sYw = sY + wave * 8 * P;
 
     // ---- asynchronous tile copy of one head into buffer `buf`; the per-lane source offsets do not depend on the head
     const uint32_t wave_u = uniform(wave), lds_S = uniform(lds_addr_of(sS)), lds_X = uniform(lds_addr_of(sX)), lds_LD = uniform(lds_addr_of(sLD));
@@ -185,10 +184,13 @@ ssd_y16_kernel(const DiagArgs a) {
         const T* cS = sS + buf * (P * N);
         const T* cX = sX + buf * (kQ * P);
 
-        const float off_fast = __expf(lref);
-        auto off_scale = [&](int v) -> float { return fast ? off_fast : __expf(sl[row0 + acc_row(lane, v)]); };
+        // Both products are issued with the operands swapped (the two operand register layouts are the same), so the
+        // accumulators hold the TRANSPOSED output block: lane (r, half) owns token row0 + r and, per 32-channel block j,
+        // the channels 32 j + 8 q + 4 half + 0..3 (q = 0..3).  Every row-wise quantity (decay scales, the D x term, the
+        // stores) is then lane-local.
+        const float off_sc = fast ? __expf(lref) : __expf(sl[row0 + r]);
 
-        // ---- off-diagonal term: C rows (registers) x S_prev (LDS, natural layout)
+        // ---- off-diagonal term: S_prev (LDS, natural layout) x C rows (registers)
         floatx16 acc[1][BN];
         acc_zero(acc);
 #pragma unroll
@@ -197,15 +199,13 @@ ssd_y16_kernel(const DiagArgs a) {
             for (int j = 0; j < BN; ++j) {
                 const int row = j * 32 + r;
                 const Frag<T> bf = load_frag(cS + (row * SPR_S + ((ks * 2 + half) ^ tile_swz<SPR_S>(row))) * 8);
-                mma_frag(acc[0][j], fo[ks], bf);
+                mma_frag(acc[0][j], bf, fo[ks]);
             }
         }
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const float os = off_scale(v);
+        for (int j = 0; j < BN; ++j)
 #pragma unroll
-            for (int j = 0; j < BN; ++j) acc[0][j][v] *= os;
-        }
+            for (int v = 0; v < 16; ++v) acc[0][j][v] *= off_sc;
 
         // ---- diagonal term: causal C B^T fragment scaled by the decay table along k; x through transpose reads
         const int jrow = row0 + r;
@@ -244,43 +244,34 @@ ssd_y16_kernel(const DiagArgs a) {
                 Frag<T> bf;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) { bf.v[e] = lo[e]; bf.v[4 + e] = hi[e]; }
-                mma_frag(acc[0][j], af, bf);
+                mma_frag(acc[0][j], bf, af);
             }
         }
 
-        // ---- epilogue, 8 token rows at a time: fp32 through the wave-private tile, then row-contiguous 16-byte
-        //      stores of  y = u * acc + D x  (x from the same LDS tile, row-wise)
-        constexpr int LPR = P / 8;               // lanes per output row
-        constexpr int RPP = 64 / LPR;            // rows per store pass
-        T* Yp = static_cast<T*>(a.Y) + b * a.Y_sb + t0 * a.Y_sl + h * a.Y_sh;
+        // ---- epilogue: y = u * acc + D x.  A lane and its partner (lane ^ 32) hold the two halves of each group of 8
+        //      channels of their token; swapping one 4-channel group per pair (v_permlane32_swap) leaves every lane with
+        //      whole groups of 8 consecutive channels: 16-byte stores without a pass through LDS
+        const int tok = row0 + r;
+        const float fs = fast ? wu[r] : 1.f;
+        T* Yp = static_cast<T*>(a.Y) + b * a.Y_sb + t0 * a.Y_sl + h * a.Y_sh + (int64_t)tok * a.Y_sl;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            // the final row scales of accumulator rows 8 q + 4 half + 0..3: four consecutive table entries
-            floatx4 fs = {1.f, 1.f, 1.f, 1.f};
-            if (fast) fs = *reinterpret_cast<const floatx4*>(wu + 8 * q + 4 * half);
+        for (int j = 0; j < BN; ++j) {
 #pragma unroll
-            for (int j = 0; j < BN; ++j)
+            for (int qp = 0; qp < 2; ++qp) {
+                float g8[8];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) sYw[(4 * half + e) * P + j * 32 + r] = acc[0][j][4 * q + e] * fs[e];
-            wave_lds_sync();
-#pragma unroll
-            for (int ps = 0; ps < 8 / RPP; ++ps) {
-                const int rl = ps * RPP + lane / LPR, cv = lane % LPR;
-                const int tok = row0 + 8 * q + rl;
-                const floatx4 ya = *reinterpret_cast<const floatx4*>(sYw + rl * P + cv * 8);
-                const floatx4 yb = *reinterpret_cast<const floatx4*>(sYw + rl * P + cv * 8 + 4);
-                const uint4 xr = *reinterpret_cast<const uint4*>(cX + (tok * SPR_X + (cv ^ tile_swz<SPR_X>(tok))) * 8);
+                for (int e = 0; e < 4; ++e) {
+                    pair_swap(acc[0][j][8 * qp + e], acc[0][j][8 * qp + 4 + e], g8[e], g8[4 + e]);
+                }
+                const int p0 = j * 32 + 8 * (2 * qp + half);
+                const uint4 xr = *reinterpret_cast<const uint4*>(cX + (tok * SPR_X + ((p0 >> 3) ^ tile_swz<SPR_X>(tok))) * 8);
                 const T* xe = reinterpret_cast<const T*>(&xr);
                 uint4 o;
                 T* oe = reinterpret_cast<T*>(&o);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    oe[e] = from_f32<T>(ya[e] + Dh * to_f32(xe[e]));
-                    oe[4 + e] = from_f32<T>(yb[e] + Dh * to_f32(xe[4 + e]));
-                }
-                if (tok < valid) *reinterpret_cast<uint4*>(Yp + (int64_t)tok * a.Y_sl + cv * 8) = o;
+                for (int e = 0; e < 8; ++e) oe[e] = from_f32<T>(fs * g8[e] + Dh * to_f32(xe[e]));
+                if (tok < valid) *reinterpret_cast<uint4*>(Yp + p0) = o;
             }
-            wave_lds_sync();
         }
     }
 }
