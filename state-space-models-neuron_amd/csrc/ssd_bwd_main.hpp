@@ -11,7 +11,9 @@
 //            dx = dt_j dxd + D dy,   dir_j = sum_p dxd x,   rb_j = dt_j sum_p (state part of dxd) x,
 //            dl_c[i] = e^{l_i} sum_p dy[i][p] (sum_n C[i][n] S_prev[p][n]),   dD partial = sum dy x
 //            (B rows, C rows and the transposed causal C B^T rows of its tokens stay on chip: registers, and for half of
-//            the C fragments a wave-private LDS tile)
+//            the C fragments a wave-private LDS tile).  Its MFMAs are issued with swapped operands, so a lane's
+//            accumulators belong to ONE token: scales and the row dot products are lane-local, and dx leaves in 16-byte
+//            stores after one lane-pair swap per 4-channel group, without a pass through LDS.
 //   role B (waves 4-7):  dB_off[j][n] += dt_j e^{Lam-l_j} sum_p x[j][p] dS[p][n]
 //                        dC_off[i][n] += e^{l_i}          sum_p dy[i][p] S_prev[p][n]
 //            accumulated over the workgroup's heads in registers (row scale applied in fp32 after the MFMA, so both
@@ -27,7 +29,7 @@ namespace m2 {
 template <int N> constexpr int bwd16_clds() { return N / 16 > 4 ? N / 32 : 0; }
 template <int P, int N>
 constexpr size_t bwd16_smem() {
-    return (size_t)2 * ((2 * P * N + 2 * kQ * P) * 2 + 2 * kQ * sizeof(float)) + (size_t)4 * (kQ + 32) * sizeof(float) + (size_t)4 * 8 * P * sizeof(float) +
+    return (size_t)2 * ((2 * P * N + 2 * kQ * P) * 2 + 2 * kQ * sizeof(float)) + (size_t)4 * (kQ + 32) * sizeof(float) +
            (size_t)4 * 32 * (bwd16_clds<N>() * 16 + 8) * 2 + (size_t)4 * 64 * sizeof(float);
 }
 template <typename T, int P, int N>
@@ -62,10 +64,9 @@ ssd_bwd16_kernel(const Bwd16Args a) {
     T* tiles = reinterpret_cast<T*>(smem_raw);                       // [2][ dS | S_prev | dy | x ]
     float* sLD = reinterpret_cast<float*>(tiles + 2 * TILES);        // [2][ l kQ | dt kQ ]
     float* wt_all = sLD + 2 * 2 * kQ;                                // [4 role-A waves][wv kQ | wu 32]
-    float* sY = wt_all + 4 * TAB;                                    // [4 role-A waves][8][P]
     constexpr int KCL = bwd16_clds<N>(), KCR = KSN - KCL;            // C-row fragments in LDS / in registers
     constexpr int LDC = KCL * 16 + 8;
-    T* sFC = reinterpret_cast<T*>(sY + 4 * 8 * P);                   // [4 role-A waves][32][LDC]
+    T* sFC = reinterpret_cast<T*>(wt_all + 4 * TAB);                  // [4 role-A waves][32][LDC]
     float* wsB_all = reinterpret_cast<float*>(sFC + 4 * 32 * LDC);   // [4 role-B waves][ dB-side 32 | dC-side 32 ] row scales
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -121,7 +122,6 @@ ssd_bwd16_kernel(const Bwd16Args a) {
         // =============================================================== role A: dx, dir, rb, dl_c, dD
         float* wv = wt_all + rbk * TAB;
         float* wu = wv + kQ;
-        float* sYw = sY + rbk * 8 * P;
         T* sFCw = sFC + rbk * 32 * LDC;
         Frag<T> fd[8], foB[KSN], foC[KCR];
         {
@@ -166,30 +166,29 @@ ssd_bwd16_kernel(const Bwd16Args a) {
             const T* cY = cP + P * N;
             const T* cX = cY + kQ * P;
 
-            const float off_fast = __expf(Lam - lref);
-            auto off_scale = [&](int v) -> float { return fast ? off_fast : __expf(Lam - sl[row0 + acc_row(lane, v)]); };
-            auto fin_scale = [&](int v) -> float { return fast ? wu[acc_row(lane, v)] : 1.f; };
-            // sum over this wave's channels of  t[row][p] * Z[row][p]  for its 16 accumulator rows (Z row-major tile, read
-            // at the accumulator positions by transpose reads); returns one row total per lane pair (see half_wave_reduce16)
-            auto row_dot = [&](const floatx16 (&t)[1][BN], const T* Z, float (&out)[16]) {
+            // All products below are issued with the MFMA operands swapped (the two operand register layouts are the same),
+            // so the accumulators hold TRANSPOSED output blocks: lane (r, half) owns token row0 + r and, per 32-channel
+            // block j, the channels 32 j + 8 q + 4 half + 0..3 (q = 0..3).  Row scales, row dot products, the D dy term and
+            // the stores are then lane-local (plus one exchange with the partner lane l ^ 32).
+            const int tok = row0 + r;
+            const float off_sc = fast ? __expf(Lam - lref) : __expf(Lam - sl[tok]);
+            const float fin_sc = fast ? wu[r] : 1.f;
+            // sum over this lane's channels of t[channel] * Z[tok][channel] (Z: row-major tile of token rows), both lanes of the pair
+            auto row_dot = [&](const floatx16 (&t)[1][BN], const T* Z) -> float {
+                float s = 0.f;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    float s4[4] = {0.f, 0.f, 0.f, 0.f};
-                    const int tok = row0 + 8 * q + 4 * half + tr_row;
+                for (int j = 0; j < BN; ++j)
 #pragma unroll
-                    for (int j = 0; j < BN; ++j) {
-                        const int col = j * 32 + tr_col;
-                        const tvec4 zv = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-                            (M2_LDS tvec4*)(Z + (tok * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(tok))) * 8 + (col & 7)));
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) s4[e] += t[0][j][4 * q + e] * to_f32(zv[e]);
+                    for (int q = 0; q < 4; ++q) {
+                        const int p0 = j * 32 + 8 * q;
+                        const uint2 zr = *reinterpret_cast<const uint2*>(Z + (tok * SPR_X + ((p0 >> 3) ^ tile_swz<SPR_X>(tok))) * 8 + 4 * half);
+                        s += t[0][j][4 * q + 0] * unpack_lo<T>(zr.x) + t[0][j][4 * q + 1] * unpack_hi<T>(zr.x) +
+                             t[0][j][4 * q + 2] * unpack_lo<T>(zr.y) + t[0][j][4 * q + 3] * unpack_hi<T>(zr.y);
                     }
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) out[4 * q + e] = s4[e];
-                }
+                return s + __shfl_xor(s, 32, 64);
             };
 
-            // ---- dl_c: (C rows x S_prev) . dy, row scale e^{l_i}
+            // ---- dl_c[i] = e^{l_i} sum_p dy[i][p] (sum_n C[i][n] S_prev[p][n])
             {
                 floatx16 yo[1][BN];
                 acc_zero(yo);
@@ -199,19 +198,15 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                     for (int j = 0; j < BN; ++j) {
                         const int row = j * 32 + r;
                         const Frag<T> bf = load_frag(cP + (row * SPR_S + ((ks * 2 + half) ^ tile_swz<SPR_S>(row))) * 8);
-                        mma_frag(yo[0][j], ks < KCR ? foC[ks < KCR ? ks : 0] : load_frag(sFCw + r * LDC + (ks - KCR) * 16 + half * 8), bf);
+                        mma_frag(yo[0][j], bf, ks < KCR ? foC[ks < KCR ? ks : 0] : load_frag(sFCw + r * LDC + (ks - KCR) * 16 + half * 8));
                     }
                 }
-                float dv[16];
-                row_dot(yo, cY, dv);
-                int ri;
-                const float tot = half_wave_reduce16(dv, &ri);
-                const int row = row0 + acc_row(lane, ri);          // the row scale is applied to the row total
-                if ((lane & 1) == 0) a.dlc[bhc * kQ + row] = row < valid ? tot * __expf(sl[row]) : 0.f;
+                const float tot = row_dot(yo, cY);
+                if (half == 0) a.dlc[bhc * kQ + tok] = tok < valid ? tot * __expf(sl[tok]) : 0.f;
             }
 
             __builtin_amdgcn_sched_barrier(0);
-            // ---- state part of dxd: B rows (registers) x dS (LDS, natural layout)
+            // ---- state part of dxd: dS (LDS, natural layout) x B rows (registers)
             floatx16 acc[1][BN];
             acc_zero(acc);
 #pragma unroll
@@ -220,24 +215,18 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                 for (int j = 0; j < BN; ++j) {
                     const int row = j * 32 + r;
                     const Frag<T> bf = load_frag(cS + (row * SPR_S + ((ks * 2 + half) ^ tile_swz<SPR_S>(row))) * 8);
-                    mma_frag(acc[0][j], foB[ks], bf);
+                    mma_frag(acc[0][j], bf, foB[ks]);
                 }
             }
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const float os = off_scale(v);
+            for (int j = 0; j < BN; ++j)
 #pragma unroll
-                for (int j = 0; j < BN; ++j) acc[0][j][v] *= os;
-            }
+                for (int v = 0; v < 16; ++v) acc[0][j][v] *= off_sc;
             __builtin_amdgcn_sched_barrier(0);
             // ---- rb_j = dt_j sum_p x[j][p] * (state part, final scale applied)
             {
-                float rv[16];
-                row_dot(acc, cX, rv);
-                int ri;
-                const float tot = half_wave_reduce16(rv, &ri);
-                const int row = row0 + acc_row(lane, ri);
-                if ((lane & 1) == 0) a.rbp[bhc * kQ + row] = tot * fin_scale(ri) * sd[row];
+                const float tot = row_dot(acc, cX);
+                if (half == 0) a.rbp[bhc * kQ + tok] = tot * fin_sc * sd[tok];
             }
 
             __builtin_amdgcn_sched_barrier(0);
@@ -261,8 +250,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                     }
                 }
                 keep_packed(fd[ks]);
-                keep_packed(fd[ks]);
-            const Frag<T> af = scale_frag(fd[ks], f);
+                const Frag<T> af = scale_frag(fd[ks], f);
 #pragma unroll
                 for (int j = 0; j < BN; ++j) {
                     const int col = j * 32 + tr_col;
@@ -274,61 +262,45 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                     Frag<T> bf;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) { bf.v[e] = lo[e]; bf.v[4 + e] = hi[e]; }
-                    mma_frag(acc[0][j], af, bf);
+                    mma_frag(acc[0][j], bf, af);
                 }
             }
 
             __builtin_amdgcn_sched_barrier(0);
-            // ---- epilogue, 8 token rows at a time: fp32 through the wave-private tile, then row-wise
-            constexpr int LPR = P / 8;               // lanes per output row
-            constexpr int RPP = 64 / LPR;            // rows per pass
-            static_assert(RPP <= 8 && 8 % RPP == 0, "row passes");
-            T* dXp = static_cast<T*>(a.dx) + b * a.dx_sb + t0 * a.dx_sl + h * a.dx_sh;
-            float dD_loc = 0.f;
+            // ---- epilogue: dx = dt_j dxd + D dy, dir_j = sum_p dxd x, dD partial = sum dy x.  One lane-pair swap per
+            //      4-channel group leaves every lane with whole groups of 8 consecutive channels of its token: 16-byte
+            //      reads of x and dy, 16-byte stores of dx, no pass through LDS
+            T* dXp = static_cast<T*>(a.dx) + b * a.dx_sb + t0 * a.dx_sl + h * a.dx_sh + (int64_t)tok * a.dx_sl;
+            const float dtt = sd[tok];
+            float dir = 0.f, dd = 0.f;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                // the final row scales of accumulator rows 8 q + 4 half + 0..3: four consecutive table entries
-                floatx4 fs = {1.f, 1.f, 1.f, 1.f};
-                if (fast) fs = *reinterpret_cast<const floatx4*>(wu + 8 * q + 4 * half);
+            for (int j = 0; j < BN; ++j) {
 #pragma unroll
-                for (int j = 0; j < BN; ++j)
+                for (int qp = 0; qp < 2; ++qp) {
+                    float g8[8];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) sYw[(4 * half + e) * P + j * 32 + r] = acc[0][j][4 * q + e] * fs[e];
-                wave_lds_sync();
-#pragma unroll
-                for (int ps = 0; ps < 8 / RPP; ++ps) {
-                    const int rl = ps * RPP + lane / LPR, cv = lane % LPR;
-                    const int tok = row0 + 8 * q + rl;
-                    const floatx4 ya = *reinterpret_cast<const floatx4*>(sYw + rl * P + cv * 8);
-                    const floatx4 yb = *reinterpret_cast<const floatx4*>(sYw + rl * P + cv * 8 + 4);
-                    const int slot = cv ^ tile_swz<SPR_X>(tok);
+                    for (int e = 0; e < 4; ++e) pair_swap(acc[0][j][8 * qp + e], acc[0][j][8 * qp + 4 + e], g8[e], g8[4 + e]);
+                    const int p0 = j * 32 + 8 * (2 * qp + half);
+                    const int slot = (p0 >> 3) ^ tile_swz<SPR_X>(tok);
                     const uint4 xr = *reinterpret_cast<const uint4*>(cX + (tok * SPR_X + slot) * 8);
                     const uint4 gr = *reinterpret_cast<const uint4*>(cY + (tok * SPR_X + slot) * 8);
-                    const T* xe = reinterpret_cast<const T*>(&xr);
-                    const T* ge = reinterpret_cast<const T*>(&gr);
-                    const float dtt = sd[tok];
-                    uint4 ov;
-                    T* oe = reinterpret_cast<T*>(&ov);
-                    float dir = 0.f, dd = 0.f;
+                    const uint32_t xw[4] = {xr.x, xr.y, xr.z, xr.w}, gw[4] = {gr.x, gr.y, gr.z, gr.w};
+                    uint32_t ow[4];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const float dxd = e < 4 ? ya[e] : yb[e - 4];
-                        const float x_ = to_f32(xe[e]), gy = to_f32(ge[e]);
-                        oe[e] = from_f32<T>(dtt * dxd + Dh * gy);
-                        dir += dxd * x_;
-                        dd += gy * x_;
+                    for (int e = 0; e < 4; ++e) {
+                        const float d0 = fin_sc * g8[2 * e], d1 = fin_sc * g8[2 * e + 1];
+                        const float x0 = unpack_lo<T>(xw[e]), x1 = unpack_hi<T>(xw[e]);
+                        const float y0 = unpack_lo<T>(gw[e]), y1 = unpack_hi<T>(gw[e]);
+                        ow[e] = pack2<T>(dtt * d0 + Dh * y0, dtt * d1 + Dh * y1);
+                        dir += d0 * x0 + d1 * x1;
+                        dd += y0 * x0 + y1 * x1;
                     }
-                    if (tok < valid) {
-                        *reinterpret_cast<uint4*>(dXp + (int64_t)tok * a.dx_sl + cv * 8) = ov;
-                        dD_loc += dd;
-                    }
-#pragma unroll
-                    for (int m = 1; m < LPR; m <<= 1) dir += __shfl_xor(dir, m, 64);      // the LPR lanes that share the row
-                    if (cv == 0) a.dirp[bhc * kQ + tok] = dir;
+                    if (tok < valid) *reinterpret_cast<uint4*>(dXp + p0) = uint4{ow[0], ow[1], ow[2], ow[3]};
                 }
-                wave_lds_sync();
             }
-            dD_loc = warp_sum(dD_loc);
+            dir += __shfl_xor(dir, 32, 64);
+            if (half == 0) a.dirp[bhc * kQ + tok] = dir;
+            float dD_loc = warp_sum(tok < valid ? dd : 0.f);
             if (lane == 0) { a.dDp8[bhc * 8 + wave] = dD_loc; a.dDp8[bhc * 8 + wave + 4] = 0.f; }
         }
     } else {
