@@ -116,9 +116,46 @@ template <int ACT> __device__ __forceinline__ float act_grad_f(float z) {
     return 1.f;
 }
 
+// Value of lane (l ^ M) for M in {1, 2, 4, 8, 16, 32}, without the LDS crossbar (a generic shuffle is a ds_bpermute):
+// DPP quad permutes / row rotation / two masked row shifts inside a row of 16 lanes, and the row / half-wave swaps of
+// gfx950 (v_permlane16_swap, v_permlane32_swap) across rows.  All 64 lanes must be active.
+template <int CTRL, int BANK>
+__device__ __forceinline__ float dpp_move(float old, float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, x), CTRL, 0xF, BANK, false));
+}
+template <int M>
+__device__ __forceinline__ float lane_xor(float x) {
+    static_assert(M == 1 || M == 2 || M == 4 || M == 8 || M == 16 || M == 32, "lane_xor: single-bit masks");
+    if constexpr (M == 1) return dpp_move<0xB1, 0xF>(x, x);                  // quad_perm [1,0,3,2]
+    else if constexpr (M == 2) return dpp_move<0x4E, 0xF>(x, x);             // quad_perm [2,3,0,1]
+    else if constexpr (M == 4) return dpp_move<0x114, 0xA>(dpp_move<0x104, 0x5>(x, x), x);     // row_shl:4 into banks 0, 2; row_shr:4 into banks 1, 3
+    else if constexpr (M == 8) return dpp_move<0x128, 0xF>(x, x);            // row_ror:8
+    else {
+        const uint32_t u = __builtin_bit_cast(uint32_t, x);
+        uint32_t r0, r1;
+        if constexpr (M == 16) { const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false); r0 = r[0]; r1 = r[1]; }
+        else { const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false); r0 = r[0]; r1 = r[1]; }
+        // r0 = { own | partner } and r1 = { partner | own } for the lower | upper member of each pair
+        return __builtin_bit_cast(float, (threadIdx.x & M) ? r0 : r1);
+    }
+}
+// x + (value of lane l ^ M): for the two swap masks both outputs of the swap are simply added
+template <int M>
+__device__ __forceinline__ float lane_xor_add(float x) {
+    if constexpr (M == 16 || M == 32) {
+        const uint32_t u = __builtin_bit_cast(uint32_t, x);
+        uint32_t r0, r1;
+        if constexpr (M == 16) { const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false); r0 = r[0]; r1 = r[1]; }
+        else { const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false); r0 = r[0]; r1 = r[1]; }
+        return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+    } else {
+        return x + lane_xor<M>(x);
+    }
+}
+
 __device__ __forceinline__ float warp_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    v = lane_xor_add<32>(v); v = lane_xor_add<16>(v); v = lane_xor_add<8>(v);
+    v = lane_xor_add<4>(v); v = lane_xor_add<2>(v); v = lane_xor_add<1>(v);
     return v;
 }
 

@@ -355,8 +355,8 @@ conv_reduce_partials_kernel(const float* __restrict__ part, int64_t nslots, int6
 #pragma unroll 4
         for (int64_t r = q; r < nslots; r += 4) s += part[(r * C + c) * kk + i];
     }
-    s += __shfl_xor(s, 1, 64);
-    s += __shfl_xor(s, 2, 64);
+    s = lane_xor_add<1>(s);
+    s = lane_xor_add<2>(s);
     if (!live || q != 0) return;
     if (i < k) st_param(dw, pd, c * k + i, s);
     else if (db) st_param(db, pd, c, s);

@@ -91,6 +91,17 @@ decode_conv_vec_kernel(const bf16_t* __restrict__ xBC, bf16_t* __restrict__ conv
 
 // VEC = 4: n % 4 == 0, float4 accesses; VEC = 1: any n.
 // GL lanes (a power of two <= 64) share one state row; rows per pass = 256 / GL.
+// sum over each group of GL adjacent lanes (GL a power of two, wave-uniform; all lanes active)
+__device__ __forceinline__ float group_sum(float v, int GL) {
+    if (GL > 32) v = lane_xor_add<32>(v);
+    if (GL > 16) v = lane_xor_add<16>(v);
+    if (GL > 8) v = lane_xor_add<8>(v);
+    if (GL > 4) v = lane_xor_add<4>(v);
+    if (GL > 2) v = lane_xor_add<2>(v);
+    if (GL > 1) v = lane_xor_add<1>(v);
+    return v;
+}
+
 template <typename T, int VEC>
 __global__ void __launch_bounds__(256)
 decode_ssm_kernel(float* __restrict__ S, const float* __restrict__ act, const T* __restrict__ dt, const float* __restrict__ A,
@@ -130,7 +141,7 @@ decode_ssm_kernel(float* __restrict__ S, const float* __restrict__ act, const T*
 #pragma unroll
                 for (int q = 0; q < 4; ++q) { sv[u][q] = sv[u][q] * dA + dx * bv[q]; part += sv[u][q] * cv[q]; }
                 __builtin_nontemporal_store(sv[u], reinterpret_cast<floatx4*>(Sp + (int64_t)pp * N + sub * 4));
-                for (int off = GL >> 1; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+                part = group_sum(part, GL);
                 if (sub == 0) y[b * ysb + h * P + pp] = from_f32<T>(part + Dh * xv[u]);
             }
         }
@@ -158,7 +169,7 @@ decode_ssm_kernel(float* __restrict__ S, const float* __restrict__ act, const T*
                 }
             }
         }
-        for (int off = GL >> 1; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+        part = group_sum(part, GL);
         if (pp < P && sub == 0) y[b * ysb + h * P + pp] = from_f32<T>(part + Dh * xv);
     }
 }

@@ -223,23 +223,23 @@ __device__ __forceinline__ float half_wave_reduce16(float (&v)[16], int* reg_ind
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
         const float keep = b4 ? v[k + 8] : v[k], send = b4 ? v[k] : v[k + 8];
-        v[k] = keep + __shfl_xor(send, 16, 64);
+        v[k] = keep + lane_xor<16>(send);
     }
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const float keep = b3 ? v[k + 4] : v[k], send = b3 ? v[k] : v[k + 4];
-        v[k] = keep + __shfl_xor(send, 8, 64);
+        v[k] = keep + lane_xor<8>(send);
     }
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
         const float keep = b2 ? v[k + 2] : v[k], send = b2 ? v[k] : v[k + 2];
-        v[k] = keep + __shfl_xor(send, 4, 64);
+        v[k] = keep + lane_xor<4>(send);
     }
     {
         const float keep = b1 ? v[1] : v[0], send = b1 ? v[0] : v[1];
-        v[0] = keep + __shfl_xor(send, 2, 64);
+        v[0] = keep + lane_xor<2>(send);
     }
-    v[0] += __shfl_xor(v[0], 1, 64);
+    v[0] = lane_xor_add<1>(v[0]);
     *reg_index = (b4 ? 8 : 0) + (b3 ? 4 : 0) + (b2 ? 2 : 0) + (b1 ? 1 : 0);
     return v[0];
 }

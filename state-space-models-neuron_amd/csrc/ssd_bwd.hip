@@ -162,7 +162,7 @@ dg_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
         if ((lane & 1) == 0) s_rs[(wave & 1) * kQ + rb * 32 + acc_row(lane, ri)] = rtot;
 #pragma unroll
         for (int jb = 0; jb < 2; ++jb) {
-            const float cs = csum[jb] + __shfl_xor(csum[jb], 32, 64);
+            const float cs = lane_xor_add<32>(csum[jb]);
             if (lane < 32) s_cs[rb * kQ + (cb0 + jb) * 32 + lane] = cs;
         }
         __syncthreads();

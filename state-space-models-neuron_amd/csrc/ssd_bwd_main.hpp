@@ -185,7 +185,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                         s += t[0][j][4 * q + 0] * unpack_lo<T>(zr.x) + t[0][j][4 * q + 1] * unpack_hi<T>(zr.x) +
                              t[0][j][4 * q + 2] * unpack_lo<T>(zr.y) + t[0][j][4 * q + 3] * unpack_hi<T>(zr.y);
                     }
-                return s + __shfl_xor(s, 32, 64);
+                return lane_xor_add<32>(s);
             };
 
             // ---- dl_c[i] = e^{l_i} sum_p dy[i][p] (sum_n C[i][n] S_prev[p][n])
@@ -298,7 +298,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                     if (tok < valid) *reinterpret_cast<uint4*>(dXp + p0) = uint4{ow[0], ow[1], ow[2], ow[3]};
                 }
             }
-            dir += __shfl_xor(dir, 32, 64);
+            dir = lane_xor_add<32>(dir);
             if (half == 0) a.dirp[bhc * kQ + tok] = dir;
             float dD_loc = warp_sum(tok < valid ? dd : 0.f);
             if (lane == 0) { a.dDp8[bhc * 8 + wave] = dD_loc; a.dDp8[bhc * 8 + wave + 4] = 0.f; }

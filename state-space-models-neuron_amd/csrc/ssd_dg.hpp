@@ -183,7 +183,7 @@ dg16_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
         int ri;
         const float rtot = half_wave_reduce16(rsum, &ri);
         if ((lane & 1) == 0) s_rs[cb * kQ + rb * 32 + acc_row(lane, ri)] = rtot;
-        csum += __shfl_xor(csum, 32, 64);
+        csum = lane_xor_add<32>(csum);
         if (lane < 32) s_cs[rb * kQ + cb * 32 + lane] = csum;
     }
     __syncthreads();

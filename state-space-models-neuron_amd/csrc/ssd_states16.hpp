@@ -83,6 +83,8 @@ state_pass16_kernel(const StatePassArgs a) {
     const int tr_col = ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
     typedef T tvec4 __attribute__((ext_vector_type(4)));
 
+    // The MFMAs are issued with swapped operands: acc[i][j][v] is the state at row pw P/2 + 32 i + r, column
+    // n0 + 32 j + acc_row(lane, v), i.e. a lane holds groups of 4 consecutive columns of ONE row (8-byte staging writes).
     floatx16 acc[PBW][NBW];
 #pragma unroll
     for (int i = 0; i < PBW; ++i)
@@ -90,7 +92,7 @@ state_pass16_kernel(const StatePassArgs a) {
         for (int j = 0; j < NBW; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int row = pw * (P / 2) + i * 32 + acc_row(lane, v), col = n0 + j * 32 + r;
+                const int row = pw * (P / 2) + i * 32 + r, col = n0 + j * 32 + acc_row(lane, v);
                 acc[i][j][v] = a.init ? a.init[bh * (P * N) + row * N + col] : 0.f;
             }
 
@@ -177,7 +179,10 @@ state_pass16_kernel(const StatePassArgs a) {
 #pragma unroll
             for (int j = 0; j < NBW; ++j)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) sOw[(i * 32 + acc_row(lane, v)) * LDO + j * 32 + r] = from_f32<T>(acc[i][j][v]);
+                for (int q = 0; q < 4; ++q) {
+                    const uint2 w = {pack2<T>(acc[i][j][4 * q], acc[i][j][4 * q + 1]), pack2<T>(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3])};
+                    *reinterpret_cast<uint2*>(sOw + (i * 32 + r) * LDO + j * 32 + 8 * q + 4 * half) = w;
+                }
         wave_lds_sync();
         char* op = reinterpret_cast<char*>(static_cast<T*>(a.prev) + ((b * nc + c) * a.nheads + h) * (int64_t)(P * N));
         float dot = 0.f;
@@ -202,7 +207,7 @@ state_pass16_kernel(const StatePassArgs a) {
         }
         wave_lds_sync();
 
-        // ---- S = e^{Lam} S + X_scaled^T M
+        // ---- S = e^{Lam} S + X_scaled^T M  (accumulated as its transpose M^T X_scaled)
 #pragma unroll
         for (int i = 0; i < PBW; ++i)
 #pragma unroll
@@ -223,7 +228,7 @@ state_pass16_kernel(const StatePassArgs a) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) { af.v[e] = lo[e]; af.v[4 + e] = hi[e]; }
 #pragma unroll
-                for (int j = 0; j < NBW; ++j) mma_frag(acc[i][j], af, bf[j][ks]);
+                for (int j = 0; j < NBW; ++j) mma_frag(acc[i][j], bf[j][ks], af);
             }
         }
     };
@@ -253,7 +258,7 @@ state_pass16_kernel(const StatePassArgs a) {
             for (int j = 0; j < NBW; ++j)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const int row = pw * (P / 2) + i * 32 + acc_row(lane, v), col = n0 + j * 32 + r;
+                    const int row = pw * (P / 2) + i * 32 + r, col = n0 + j * 32 + acc_row(lane, v);
                     a.final_out[bh * (P * N) + row * N + col] = acc[i][j][v];
                 }
     }
