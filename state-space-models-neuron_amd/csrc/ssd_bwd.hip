@@ -340,9 +340,6 @@ tail1_kernel(const DaArgs d, const int64_t n_da, const SliceSumArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------
-// Group-level finish: dG = sum of the slice partials; dC = dG B + sum dCoff;  dB = dG^T C + sum dBoff.
-// grid (nchunks, ngroups, batch), 512 threads.  The head-summed dG is rounded to the operand type only here; for
-// bf16 it is split into hi + lo (two MFMA passes) so the contractions see it at ~2^-17 relative.
 // acc[0][j] += A[rows 0..31, k0:k1] * M[column blocks nb0 + j, k0:k1]^T with A in LDS (row-major) and M a transposed
 // B / C tile in MFMA operand order (mt_offset), copied to LDS as it lies: a wave's B-operand fragment is one
 // contiguous KiB.
@@ -358,16 +355,20 @@ __device__ __forceinline__ void wave_mma_mt(floatx16 (&acc)[1][NB], const T* __r
     }
 }
 
+// Group-level finish, one side per workgroup of 512 threads:  dC = dG B + sum dCoff  or  dB = dG^T C + sum dBoff  (dG and
+// the off parts already summed over the head slices).  The head-summed dG is rounded to the operand type only here; for
+// bf16 it is split into hi + lo (two MFMA passes) so the contractions see it at ~2^-17 relative.
 template <typename T, int N>
 __device__ __forceinline__ void
 bc_final_body(const float* __restrict__ dGp, const float* __restrict__ dCp, const float* __restrict__ dBp,
               const T* __restrict__ Bt, const T* __restrict__ Ct, T* __restrict__ dB, T* __restrict__ dC,
               int64_t seqlen, int64_t ngroups, int64_t nchunks,
-              int64_t dBsb, int64_t dBsl, int64_t dBsg, int64_t dCsb, int64_t dCsl, int64_t dCsg, int64_t c, int64_t g, int64_t b) {
+              int64_t dBsb, int64_t dBsl, int64_t dBsg, int64_t dCsb, int64_t dCsl, int64_t dCsg, int64_t c, int64_t g, int64_t b,
+              const bool side_b) {
     constexpr int LDQ = lds_ld<T>(kQ);
     constexpr int NB = N / 64;
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    T* sA2 = reinterpret_cast<T*>(smem_raw);       // [kQ][LDQ]  dG (or its transpose)
+    T* sA2 = reinterpret_cast<T*>(smem_raw);       // [kQ][LDQ]  dG (dC side) or its transpose (dB side)
     T* sT2 = sA2 + kQ * LDQ;                       // [N][LDQ]   Bt or Ct
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 31;
@@ -376,13 +377,12 @@ bc_final_body(const float* __restrict__ dGp, const float* __restrict__ dCp, cons
     const int rb = wave >> 1, cb0 = (wave & 1) * 2, nb0 = (wave & 1) * NB;
     const int64_t grp = (b * nchunks + c) * ngroups + g;
 
-    // inputs are already summed over the head slices (slice_sum_kernel)
-    floatx16 dG[1][2], aC[1][NB], aB[1][NB];
+    // inputs are already summed over the head slices (slice_sum_body)
+    floatx16 dG[1][2], acc[1][NB];
     acc_zero(dG);
     {
         const float* gp = dGp + grp * (int64_t)(kQ * kQ);
-        const float* cp = dCp + grp * (int64_t)(kQ * N);
-        const float* bp = dBp + grp * (int64_t)(kQ * N);
+        const float* op = (side_b ? dBp : dCp) + grp * (int64_t)(kQ * N);
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int row = rb * 32 + acc_row(lane, v);
@@ -390,22 +390,19 @@ bc_final_body(const float* __restrict__ dGp, const float* __restrict__ dCp, cons
             for (int jb = 0; jb < 2; ++jb)
                 if (cb0 + jb <= rb) dG[0][jb][v] = gp[row * kQ + (cb0 + jb) * 32 + r];
 #pragma unroll
-            for (int jn = 0; jn < NB; ++jn) {
-                aC[0][jn][v] = cp[row * N + (nb0 + jn) * 32 + r];
-                aB[0][jn][v] = bp[row * N + (nb0 + jn) * 32 + r];
-            }
+            for (int jn = 0; jn < NB; ++jn) acc[0][jn][v] = op[row * N + (nb0 + jn) * 32 + r];
         }
     }
     constexpr int NPASS = sizeof(T) == 2 ? 2 : 1;
-    // dC[i][n] += sum_{j<=i} dG[i][j] B[j][n]
-    auto stage_mt = [&](const T* tile) {
-        if constexpr (sizeof(T) == 2) {
-            for (int e = tid; e < N * kQ / 8; e += 512) *reinterpret_cast<uint4*>(sT2 + e * 8) = *reinterpret_cast<const uint4*>(tile + e * 8);
-        } else {
-            stage_rows<T, N, kQ, 512, false>(sT2, LDQ, tile, kQ, N, nullptr, tid);
-        }
-    };
-    stage_mt(Bt + grp * (int64_t)(N * kQ));
+    //   dC[i][n] += sum_{j<=i} dG[i][j] B[j][n]      (A = dG,   k = j in [0, 32 (rb + 1)) )
+    //   dB[j][n] += sum_{i>=j} dG[i][j] C[i][n]      (A = dG^T, k = i in [32 rb, kQ) )
+    const T* tile = (side_b ? Ct : Bt) + grp * (int64_t)(N * kQ);
+    if constexpr (sizeof(T) == 2) {
+        for (int e = tid; e < N * kQ / 8; e += 512) *reinterpret_cast<uint4*>(sT2 + e * 8) = *reinterpret_cast<const uint4*>(tile + e * 8);
+    } else {
+        stage_rows<T, N, kQ, 512, false>(sT2, LDQ, tile, kQ, N, nullptr, tid);
+    }
+    const int k0 = side_b ? rb * 32 : 0, k1 = side_b ? kQ : (rb + 1) * 32;
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
 #pragma unroll
@@ -415,42 +412,21 @@ bc_final_body(const float* __restrict__ dGp, const float* __restrict__ dCp, cons
                 const int i = rb * 32 + acc_row(lane, v), j = (cb0 + jb) * 32 + r;
                 const float full = dG[0][jb][v];
                 const T hi = from_f32<T>(full);
-                sA2[i * LDQ + j] = pass == 0 ? hi : from_f32<T>(full - to_f32(hi));
+                sA2[side_b ? j * LDQ + i : i * LDQ + j] = pass == 0 ? hi : from_f32<T>(full - to_f32(hi));
             }
         __syncthreads();
-        if constexpr (sizeof(T) == 2) wave_mma_mt<NB>(aC, sA2 + rb * 32 * LDQ, LDQ, sT2, nb0, 0, (rb + 1) * 32);
-        else wave_mma<1, NB>(aC, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, 0, (rb + 1) * 32);
+        if constexpr (sizeof(T) == 2) wave_mma_mt<NB>(acc, sA2 + rb * 32 * LDQ, LDQ, sT2, nb0, k0, k1);
+        else wave_mma<1, NB>(acc, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, k0, k1);
         __syncthreads();
     }
-    // dB[j][n] += sum_{i>=j} dG[i][j] C[i][n]
-    stage_mt(Ct + grp * (int64_t)(N * kQ));
-#pragma unroll
-    for (int pass = 0; pass < NPASS; ++pass) {
-#pragma unroll
-        for (int jb = 0; jb < 2; ++jb)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int i = rb * 32 + acc_row(lane, v), j = (cb0 + jb) * 32 + r;
-                const float full = dG[0][jb][v];
-                const T hi = from_f32<T>(full);
-                sA2[j * LDQ + i] = pass == 0 ? hi : from_f32<T>(full - to_f32(hi));
-            }
-        __syncthreads();
-        if constexpr (sizeof(T) == 2) wave_mma_mt<NB>(aB, sA2 + rb * 32 * LDQ, LDQ, sT2, nb0, rb * 32, kQ);
-        else wave_mma<1, NB>(aB, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, rb * 32, kQ);
-        __syncthreads();
-    }
-    T* dBo = dB + b * dBsb + t0 * dBsl + g * dBsg;
-    T* dCo = dC + b * dCsb + t0 * dCsl + g * dCsg;
+    T* out = side_b ? dB + b * dBsb + t0 * dBsl + g * dBsg : dC + b * dCsb + t0 * dCsl + g * dCsg;
+    const int64_t osl = side_b ? dBsl : dCsl;
 #pragma unroll
     for (int jn = 0; jn < NB; ++jn)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int row = rb * 32 + acc_row(lane, v), col = (nb0 + jn) * 32 + r;
-            if (row < valid) {
-                dCo[(int64_t)row * dCsl + col] = from_f32<T>(aC[0][jn][v]);
-                dBo[(int64_t)row * dBsl + col] = from_f32<T>(aB[0][jn][v]);
-            }
+            if (row < valid) out[(int64_t)row * osl + col] = from_f32<T>(acc[0][jn][v]);
         }
 }
 
@@ -477,8 +453,9 @@ __device__ __forceinline__ void ad_reduce_body(const float* __restrict__ dAp, co
     }
 }
 
-// The group-level finish and the per-head reductions in one launch: the first n_bc workgroups run bc_final_body for
-// (chunk, group, batch) = the index split in that order, the others ad_reduce_body for one head each.
+// The group-level finish and the per-head reductions in one launch: the first 2 n_bc workgroups run bc_final_body for
+// (side, chunk, group, batch) = the index split in that order (side 0: dC, side 1: dB -- two independent products,
+// so two workgroups), the others ad_reduce_body for one head each.
 struct Tail2Args {
     const float* dGp; const float* dCp; const float* dBp; const void* Bt; const void* Ct; void* dB; void* dC;
     int64_t dBsb, dBsl, dBsg, dCsb, dCsl, dCsg;
@@ -489,12 +466,14 @@ template <typename T, int N>
 __global__ void __launch_bounds__(512)
 tail2_kernel(const Tail2Args a) {
     const int64_t blk = blockIdx.x;
-    if (blk < a.n_bc) {
-        const int64_t c = blk % a.nchunks, g = (blk / a.nchunks) % a.ngroups, b = blk / (a.nchunks * a.ngroups);
+    if (blk < 2 * a.n_bc) {
+        const int64_t q = blk >> 1;
+        const int64_t c = q % a.nchunks, g = (q / a.nchunks) % a.ngroups, b = q / (a.nchunks * a.ngroups);
         bc_final_body<T, N>(a.dGp, a.dCp, a.dBp, static_cast<const T*>(a.Bt), static_cast<const T*>(a.Ct), static_cast<T*>(a.dB),
-                            static_cast<T*>(a.dC), a.seqlen, a.ngroups, a.nchunks, a.dBsb, a.dBsl, a.dBsg, a.dCsb, a.dCsl, a.dCsg, c, g, b);
+                            static_cast<T*>(a.dC), a.seqlen, a.ngroups, a.nchunks, a.dBsb, a.dBsl, a.dBsg, a.dCsb, a.dCsl, a.dCsg, c, g, b,
+                            (blk & 1) != 0);
     } else {
-        ad_reduce_body(a.dAp, a.dDp, a.dA, a.dD, a.batch, a.nheads, a.nchunks, blk - a.n_bc);
+        ad_reduce_body(a.dAp, a.dDp, a.dA, a.dD, a.batch, a.nheads, a.nchunks, blk - 2 * a.n_bc);
     }
 }
 
@@ -672,7 +651,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         ta.dCsb = p->dC_stride_b; ta.dCsl = p->dC_stride_l; ta.dCsg = p->dC_stride_g;
         ta.dAp = w.dAp; ta.dDp = w.dDp; ta.dA = p->dA; ta.dD = p->D ? p->dD : nullptr;
         ta.seqlen = p->seqlen; ta.ngroups = p->ngroups; ta.nchunks = nc; ta.batch = p->batch; ta.nheads = p->nheads; ta.n_bc = ngrp;
-        k<<<(unsigned)(ngrp + p->nheads), 512, sm, st>>>(ta);
+        k<<<(unsigned)(2 * ngrp + p->nheads), 512, sm, st>>>(ta);
         if ((rc = check_launch("ssd tail2_kernel"))) return rc;
     }
     return M2_OK;

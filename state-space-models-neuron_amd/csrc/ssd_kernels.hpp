@@ -32,8 +32,9 @@ namespace m2 {
 //   Gmt [kQ][kQ] T               its transpose: Gmt[j][i] = G[i][j] for i >= j (backward dx term, rows j)
 //   Bt, Ct N x kQ T              B and C transposed (tokens contiguous), laid out by mt_offset: MFMA operands of the
 //                                chunk-state products
-// One workgroup of 256 threads per (chunk, group, batch).  The upper-right 64x64 quadrant of G is never consumed and is
-// neither computed nor written.
+// Two workgroups of 256 threads per (chunk, group, batch): one for G and its two operand-type copies, one for the
+// transposed tiles (independent work on the same inputs).  The upper-right 64x64 quadrant of G is never consumed and
+// is neither computed nor written.
 // Element offset of the 8 tokens s0 .. s0 + 7 (s0 a multiple of 8) of state column n inside a transposed B / C tile.
 //   fp32   : [N][kQ], tokens contiguous (rows staged into LDS by chunk_state_kernel);
 //   16-bit : MFMA operand order [N / 32][kQ / 16][64 lanes][8]: the B-operand fragment of a wave for column block n / 32
@@ -50,7 +51,8 @@ __device__ __forceinline__ void
 cb_body(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict__ Gf, T* __restrict__ Gm, T* __restrict__ Gmt,
         T* __restrict__ Bt, T* __restrict__ Ct,
         int64_t seqlen, int64_t ngroups, int64_t nchunks,
-        int64_t Bsb, int64_t Bsl, int64_t Bsg, int64_t Csb, int64_t Csl, int64_t Csg, int64_t c, int64_t g, int64_t b) {
+        int64_t Bsb, int64_t Bsl, int64_t Bsg, int64_t Csb, int64_t Csl, int64_t Csg, int64_t c, int64_t g, int64_t b,
+        const bool transposes) {
     constexpr int KB = 64;
     constexpr int LD = lds_ld<T>(KB);
     constexpr int V = VecTraits<T>::kVec;
@@ -72,9 +74,9 @@ cb_body(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict__ 
         stage_rows<T, kQ, KB, 256, false>(sC, LD, Cp + k0, Csl, valid, nullptr, tid);
         stage_rows<T, kQ, KB, 256, false>(sB, LD, Bp + k0, Bsl, valid, nullptr, tid);
         __syncthreads();
-        if (!(wm == 0 && wn == 1)) wave_mma<2, 2>(acc, sC + wm * 64 * LD, LD, sB + wn * 64 * LD, LD, 0, KB);
+        if (!transposes && !(wm == 0 && wn == 1)) wave_mma<2, 2>(acc, sC + wm * 64 * LD, LD, sB + wn * 64 * LD, LD, 0, KB);
         // transposed copies of this 64-column slab: thread -> (state column n, group of V tokens)
-        for (int e = tid; e < KB * (kQ / V); e += 256) {
+        for (int e = tid; transposes && e < KB * (kQ / V); e += 256) {
             const int n = e % KB, s0 = (e / KB) * V;
             T vb[V], vc[V];
 #pragma unroll
@@ -84,7 +86,7 @@ cb_body(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict__ 
         }
         __syncthreads();
     }
-    if (wm == 0 && wn == 1) return;
+    if (transposes || (wm == 0 && wn == 1)) return;
     float* Gfp = Gf + grp * (int64_t)(kQ * kQ);
     T* Gmp = Gm + grp * (int64_t)(kQ * kQ);
     T* Gmtp = Gmt + grp * (int64_t)(kQ * kQ);
@@ -135,7 +137,7 @@ ld_table_body(const void* __restrict__ dt, int dt_f32, const float* __restrict__
 }
 
 // Both preparations in one launch (they are independent, and either alone leaves most of the GPU idle): the first
-// n_cb workgroups run cb_body for (chunk, group, batch) = the index split in that order, the others ld_table_body.
+// 2 n_cb workgroups run cb_body for (part, chunk, group, batch) = the index split in that order, the others ld_table_body.
 struct PrepArgs {
     const void* Bm; const void* Cm; float* Gf; void* Gm; void* Gmt; void* Bt; void* Ct;
     int64_t Bsb, Bsl, Bsg, Csb, Csl, Csg;
@@ -146,13 +148,14 @@ template <typename T, int N>
 __global__ void __launch_bounds__(256)
 prep_kernel(const PrepArgs a) {
     const int64_t blk = blockIdx.x;
-    if (blk < a.n_cb) {
-        const int64_t c = blk % a.nchunks, g = (blk / a.nchunks) % a.ngroups, b = blk / (a.nchunks * a.ngroups);
+    if (blk < 2 * a.n_cb) {
+        const int64_t q = blk >> 1;
+        const int64_t c = q % a.nchunks, g = (q / a.nchunks) % a.ngroups, b = q / (a.nchunks * a.ngroups);
         cb_body<T, N>(static_cast<const T*>(a.Bm), static_cast<const T*>(a.Cm), a.Gf, static_cast<T*>(a.Gm), static_cast<T*>(a.Gmt),
                       static_cast<T*>(a.Bt), static_cast<T*>(a.Ct), a.seqlen, a.ngroups, a.nchunks,
-                      a.Bsb, a.Bsl, a.Bsg, a.Csb, a.Csl, a.Csg, c, g, b);
+                      a.Bsb, a.Bsl, a.Bsg, a.Csb, a.Csl, a.Csg, c, g, b, (blk & 1) != 0);
     } else {
-        ld_table_body<T>(a.dt, a.dt_f32, a.A, a.ldtab, a.lam, a.seqlen, a.nheads, a.nchunks, a.total_bhc, a.dtsb, a.dtsl, blk - a.n_cb);
+        ld_table_body<T>(a.dt, a.dt_f32, a.A, a.ldtab, a.lam, a.seqlen, a.nheads, a.nchunks, a.total_bhc, a.dtsb, a.dtsl, blk - 2 * a.n_cb);
     }
 }
 
