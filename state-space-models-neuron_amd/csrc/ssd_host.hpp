@@ -152,7 +152,7 @@ inline int allow_smem(K kernel, size_t bytes) {
 template <typename T, int P, int N>
 inline size_t state_smem() { return (size_t)(P + N) * lds_ld<T>(kQ) * sizeof(T); }
 template <typename T>
-inline size_t cb_smem() { return (size_t)2 * kQ * lds_ld<T>(64) * sizeof(T); }
+inline size_t cb_smem(int n) { return (size_t)2 * kQ * lds_ld<T>(n) * sizeof(T); }
 
 // Decay tables, G = C B^T (+ operand tiles), local chunk states, forward state scan.  Used by the forward and, when the
 // caller did not keep the forward's chunk_states buffer, by the backward (recompute).
@@ -167,7 +167,7 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
     {
         // decay tables and G = C B^T (+ operand tiles), one launch
         auto k = prep_kernel<T, N>;
-        const size_t sm = cb_smem<T>();
+        const size_t sm = cb_smem<T>(N);
         if ((rc = allow_smem(k, sm))) return rc;
         PrepArgs pa;
         pa.Bm = Bm; pa.Cm = Cm; pa.Gf = w.G; pa.Gm = w.Gm; pa.Gmt = w.Gmt; pa.Bt = w.Bt; pa.Ct = w.Ct;

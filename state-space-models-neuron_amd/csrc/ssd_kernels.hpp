@@ -53,7 +53,7 @@ cb_body(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict__ 
         int64_t seqlen, int64_t ngroups, int64_t nchunks,
         int64_t Bsb, int64_t Bsl, int64_t Bsg, int64_t Csb, int64_t Csl, int64_t Csg, int64_t c, int64_t g, int64_t b,
         const bool transposes) {
-    constexpr int KB = 64;
+    constexpr int KB = N;          // the whole contraction length at once: one staging phase, one barrier pair
     constexpr int LD = lds_ld<T>(KB);
     constexpr int V = VecTraits<T>::kVec;
     extern __shared__ __align__(16) unsigned char smem_raw[];
