@@ -51,12 +51,12 @@ decode_conv_kernel(const T* __restrict__ xBC, T* __restrict__ conv_state, const 
 }
 
 // bf16, k == 4, W in {3, 4}, Cx % 8 == 0: one thread owns 8 consecutive channels, whose W-column histories are
-// W*16 contiguous bytes; every access is a 16-byte vector.
-template <int W>
+// W*16 contiguous bytes; every access is a 16-byte vector, the 32 taps and 8 biases of the thread included (all loads
+// are issued before any is used).
+template <int W, typename WT>
 __global__ void __launch_bounds__(256)
-decode_conv_vec_kernel(const bf16_t* __restrict__ xBC, bf16_t* __restrict__ conv_state, const void* __restrict__ w,
-                       const void* __restrict__ bias, float* __restrict__ act, int64_t nb, int64_t Cx, int64_t xsb, int pd,
-                       int activation) {
+decode_conv_vec_kernel(const bf16_t* __restrict__ xBC, bf16_t* __restrict__ conv_state, const WT* __restrict__ w,
+                       const WT* __restrict__ bias, float* __restrict__ act, int64_t nb, int64_t Cx, int64_t xsb, int activation) {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;      // (b, c8)
     const int64_t C8 = Cx / 8;
     if (idx >= nb * C8) return;
@@ -66,6 +66,26 @@ decode_conv_vec_kernel(const bf16_t* __restrict__ xBC, bf16_t* __restrict__ conv
 #pragma unroll
     for (int i = 0; i < W; ++i) raw[i] = reinterpret_cast<const uint4*>(cs)[i];
     const uint4 xr = *reinterpret_cast<const uint4*>(xBC + b * xsb + c0);
+    constexpr int PER = 16 / (int)sizeof(WT);            // parameters per 16-byte vector
+    float wv[32], bv[8];
+#pragma unroll
+    for (int i = 0; i < 32 / PER; ++i) {
+        float tmp[PER];
+        load16<WT>(w + c0 * 4 + i * PER, tmp);
+#pragma unroll
+        for (int e = 0; e < PER; ++e) wv[i * PER + e] = tmp[e];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) bv[j] = 0.f;
+    if (bias) {
+#pragma unroll
+        for (int i = 0; i < 8 / PER; ++i) {
+            float tmp[PER];
+            load16<WT>(bias + c0 + i * PER, tmp);
+#pragma unroll
+            for (int e = 0; e < PER; ++e) bv[i * PER + e] = tmp[e];
+        }
+    }
     const bf16_t* old = reinterpret_cast<const bf16_t*>(raw);                // [8 channels][W]
     const bf16_t* xin = reinterpret_cast<const bf16_t*>(&xr);
     uint4 nw[W];
@@ -73,10 +93,10 @@ decode_conv_vec_kernel(const bf16_t* __restrict__ xBC, bf16_t* __restrict__ conv
     float out[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        float z = bias ? ld_any(bias, pd, c0 + j) : 0.f;
+        float z = bv[j];
 #pragma unroll
-        for (int i = 0; i < 3; ++i) z += ld_any(w, pd, (c0 + j) * 4 + i) * to_f32(old[j * W + (W - 3) + i]);
-        z += ld_any(w, pd, (c0 + j) * 4 + 3) * to_f32(xin[j]);
+        for (int i = 0; i < 3; ++i) z += wv[j * 4 + i] * to_f32(old[j * W + (W - 3) + i]);
+        z += wv[j * 4 + 3] * to_f32(xin[j]);
 #pragma unroll
         for (int i = 0; i + 1 < W; ++i) nst[j * W + i] = old[j * W + i + 1];
         nst[j * W + W - 1] = xin[j];
@@ -206,13 +226,22 @@ extern "C" int m2_decode_step(const m2_decode_params* p, void* stream) {
     int GL = 1;
     while (GL < 64 && GL < p->dstate / vec) GL <<= 1;
     const bool vec_conv = p->dtype == M2_BF16 && p->k == 4 && (p->W == 3 || p->W == 4) && Cx % 8 == 0 &&
-                          p->xBC_stride_b % 8 == 0 && aligned16(p->xBC) && aligned16(p->conv_state);
+                          p->xBC_stride_b % 8 == 0 && aligned16(p->xBC) && aligned16(p->conv_state) && aligned16(p->conv_w) &&
+                          aligned16(p->conv_b);
     if (vec_conv) {
         const unsigned blocks = (unsigned)ceil_div(p->batch * (Cx / 8), (int64_t)256);
         const bf16_t* xb = static_cast<const bf16_t*>(p->xBC);
         bf16_t* csb = static_cast<bf16_t*>(p->conv_state);
-        if (p->W == 3) decode_conv_vec_kernel<3><<<blocks, 256, 0, st>>>(xb, csb, p->conv_w, p->conv_b, act, p->batch, Cx, p->xBC_stride_b, p->param_dtype, p->activation);
-        else decode_conv_vec_kernel<4><<<blocks, 256, 0, st>>>(xb, csb, p->conv_w, p->conv_b, act, p->batch, Cx, p->xBC_stride_b, p->param_dtype, p->activation);
+        auto go = [&](auto kern, auto wt_tag) {
+            using WT = decltype(wt_tag);
+            kern<<<blocks, 256, 0, st>>>(xb, csb, static_cast<const WT*>(p->conv_w), static_cast<const WT*>(p->conv_b), act, p->batch, Cx,
+                                         p->xBC_stride_b, p->activation);
+        };
+        if (p->param_dtype == M2_F32) {
+            if (p->W == 3) go(decode_conv_vec_kernel<3, float>, float{}); else go(decode_conv_vec_kernel<4, float>, float{});
+        } else {
+            if (p->W == 3) go(decode_conv_vec_kernel<3, bf16_t>, bf16_t{}); else go(decode_conv_vec_kernel<4, bf16_t>, bf16_t{});
+        }
         int rc = check_launch("decode_conv_vec_kernel");
         if (rc) return rc;
     }
