@@ -21,7 +21,7 @@ constexpr int kDgWaves = 10;
 template <int P>
 constexpr int dg16_ring() { return (size_t)4 * (2 * kQ * P * 2 + 1024) + 8 * 1024 <= 160 * 1024 ? 4 : 2; }    // tile buffers
 template <int P>
-constexpr size_t dg16_smem() { return (size_t)dg16_ring<P>() * (2 * kQ * P * 2 + 2 * kQ * sizeof(float)) + (size_t)(2 * 8 * kQ) * sizeof(float); }
+constexpr size_t dg16_smem() { return (size_t)dg16_ring<P>() * (2 * kQ * P * 2 + 2 * kQ * sizeof(float)) + (size_t)(2 * 8 * kQ + kDgWaves * 32) * sizeof(float); }
 
 template <typename T, int P>
 __global__ void __launch_bounds__(kDgWaves * 64)
@@ -39,6 +39,7 @@ dg16_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
     T* tiles = reinterpret_cast<T*>(smem_raw);                         // [RING][ dY | X ]
     float* sLD = reinterpret_cast<float*>(tiles + RING * 2 * TILE);    // [RING][ l kQ | dt kQ ]
     float* s_sum = sLD + RING * 2 * kQ;                                // [2 parities][ rs 4 x kQ | cs 4 x kQ ]
+    float* su = s_sum + 2 * 8 * kQ + (threadIdx.x >> 6) * 32;          // [waves][32]: row factors of this wave's block
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 31, half = lane >> 5;
@@ -129,16 +130,20 @@ dg16_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
         const int j = cb * 32 + r;
         const float lj = sl[j], dtj = sd[j];
         const float vj = __expf(fminf(l_first - lj, kMaxRange)) * dtj;
+        // row factors: one exponential per row of the block (32 lanes), read back as four consecutive table entries per
+        // group of accumulator rows 8 q + 4 half + 0..3 -- not 16 exponentials per lane
+        if (lane < 32) su[lane] = fast ? __expf(sl[rb * 32 + lane] - l_first) : sl[rb * 32 + lane];
+        wave_lds_sync();
         float ui[16];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {      // accumulator rows 8 q + 4 half + 0..3: four consecutive table entries
-            const floatx4 l4 = *reinterpret_cast<const floatx4*>(sl + rb * 32 + 8 * q + 4 * half);
+        for (int q = 0; q < 4; ++q) {
+            const floatx4 u4 = *reinterpret_cast<const floatx4*>(su + 8 * q + 4 * half);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) ui[4 * q + e] = l4[e];
+            for (int e = 0; e < 4; ++e) ui[4 * q + e] = u4[e];
         }
         if (fast) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) ui[v] = __expf(ui[v] - l_first) * vj;      // u_i * v_j
+            for (int v = 0; v < 16; ++v) ui[v] *= vj;      // u_i * v_j
         } else {
 #pragma unroll
             for (int v = 0; v < 16; ++v) ui[v] = __expf(fminf(ui[v] - lj, 0.f)) * dtj;
