@@ -8,16 +8,17 @@
 //
 // The waves are specialised by role, two per 32-token row block (so that each role's long-lived registers are its own):
 //   role A (waves 0-3): dxd[j][p] = u_j ( e^{Lam-l_ref} sum_n B[j][n] dS[p][n] + sum_{i>=j} (G[i][j] v_i) dy[i][p] )
-//            dx = dt_j dxd + D dy,   dir_j = sum_p dxd x,   rb_j = dt_j sum_p (state part of dxd) x,
-//            dl_c[i] = e^{l_i} sum_p dy[i][p] (sum_n C[i][n] S_prev[p][n]),   dD partial = sum dy x
-//            (B rows, C rows and the transposed causal C B^T rows of its tokens stay on chip: registers, and for half of
-//            the C fragments a wave-private LDS tile).  Its MFMAs are issued with swapped operands, so a lane's
-//            accumulators belong to ONE token: scales and the row dot products are lane-local, and dx leaves in 16-byte
-//            stores after one lane-pair swap per 4-channel group, without a pass through LDS.
+//            dx = dt_j dxd + D dy,   dir_j = sum_p dxd x,   rb_j = dt_j sum_p (state part of dxd) x,   dD partial = sum dy x
+//            (B rows and the transposed causal C B^T rows of its tokens stay in registers).
 //   role B (waves 4-7):  dB_off[j][n] += dt_j e^{Lam-l_j} sum_p x[j][p] dS[p][n]
 //                        dC_off[i][n] += e^{l_i}          sum_p dy[i][p] S_prev[p][n]
 //            accumulated over the workgroup's heads in registers (row scale applied in fp32 after the MFMA, so both
-//            operands are exact copies of the inputs) and written once at the end.
+//            operands are exact copies of the inputs) and written once at the end; and, from the same product before
+//            it is accumulated,   dl_c[i] = e^{l_i} sum_n C[i][n] (sum_p dy[i][p] S_prev[p][n])
+//            (the C row of the lane's token stays in registers).
+// Every MFMA is issued with its operands swapped, so a lane's accumulators belong to ONE token: row scales and row dot
+// products are lane-local (plus one exchange with the partner lane), and dx leaves in 16-byte stores after one
+// lane-pair swap per 4-channel group, without a pass through LDS.
 // The decay is factorised per row block around its LAST token (see ssd_diag.hpp), with the exact per-element
 // fallback when the block's range exceeds kMaxRange.  ddt and dA need a scan over the chunk and are left to da_body (tail1_kernel).
 #pragma once
@@ -25,12 +26,12 @@
 
 namespace m2 {
 
-// of the N / 16 C-row fragments a role-A wave needs, this many live in a wave-private LDS tile instead of registers
-template <int N> constexpr int bwd16_clds() { return N / 16 > 4 ? N / 32 : 0; }
+// of the N / 32 column blocks of a role-B lane's C row, this many are parked in LDS instead of registers
+template <int N> constexpr int bwd16_clds() { return N / 32 > 2 ? N / 64 : 0; }
 template <int P, int N>
 constexpr size_t bwd16_smem() {
     return (size_t)2 * ((2 * P * N + 2 * kQ * P) * 2 + 2 * kQ * sizeof(float)) + (size_t)4 * (kQ + 32) * sizeof(float) +
-           (size_t)4 * 32 * (bwd16_clds<N>() * 16 + 8) * 2 + (size_t)4 * 64 * sizeof(float);
+           (size_t)4 * bwd16_clds<N>() * 4 * 64 * sizeof(uint2);
 }
 template <typename T, int P, int N>
 constexpr bool bwd16_ok() { return sizeof(T) == 2 && bwd16_smem<P, N>() <= 160 * 1024; }
@@ -64,10 +65,8 @@ ssd_bwd16_kernel(const Bwd16Args a) {
     T* tiles = reinterpret_cast<T*>(smem_raw);                       // [2][ dS | S_prev | dy | x ]
     float* sLD = reinterpret_cast<float*>(tiles + 2 * TILES);        // [2][ l kQ | dt kQ ]
     float* wt_all = sLD + 2 * 2 * kQ;                                // [4 role-A waves][wv kQ | wu 32]
-    constexpr int KCL = bwd16_clds<N>(), KCR = KSN - KCL;            // C-row fragments in LDS / in registers
-    constexpr int LDC = KCL * 16 + 8;
-    T* sFC = reinterpret_cast<T*>(wt_all + 4 * TAB);                  // [4 role-A waves][32][LDC]
-    float* wsB_all = reinterpret_cast<float*>(sFC + 4 * 32 * LDC);   // [4 role-B waves][ dB-side 32 | dC-side 32 ] row scales
+    constexpr int JCL = bwd16_clds<N>(), JCR = NBN - JCL;            // C-row column blocks in LDS / in registers
+    uint2* sCw_all = reinterpret_cast<uint2*>(wt_all + 4 * TAB);     // [4 role-B waves][JCL][4][64 lanes]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 31, half = lane >> 5;
@@ -122,26 +121,21 @@ ssd_bwd16_kernel(const Bwd16Args a) {
         // =============================================================== role A: dx, dir, rb, dl_c, dD
         float* wv = wt_all + rbk * TAB;
         float* wu = wv + kQ;
-        T* sFCw = sFC + rbk * 32 * LDC;
-        Frag<T> fd[8], foB[KSN], foC[KCR];
+        Frag<T> fd[8], foB[KSN];
         {
             const T* Gp = static_cast<const T*>(a.Gmt) + ((b * a.nchunks + c) * a.ngroups + g) * (int64_t)(kQ * kQ) + (row0 + r) * kQ;
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks)
                 if (ks >= 2 * rbk) fd[ks] = load_frag(Gp + ks * 16 + half * 8);
             const T* Bp = static_cast<const T*>(a.Bm) + b * a.B_sb + (t0 + row0 + r) * a.B_sl + g * a.B_sg;
-            const T* Cp = static_cast<const T*>(a.Cm) + b * a.C_sb + (t0 + row0 + r) * a.C_sl + g * a.C_sg;
             const bool ok = row0 + r < valid;
 #pragma unroll
             for (int ks = 0; ks < KSN; ++ks) {
-                Frag<T> fc;
-                if (ok) { foB[ks] = load_frag(Bp + ks * 16 + half * 8); fc = load_frag(Cp + ks * 16 + half * 8); }
+                if (ok) foB[ks] = load_frag(Bp + ks * 16 + half * 8);
                 else {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) { foB[ks].v[e] = (T)0.f; fc.v[e] = (T)0.f; }
+                    for (int e = 0; e < 8; ++e) foB[ks].v[e] = (T)0.f;
                 }
-                if (ks < KCR) foC[ks < KCR ? ks : 0] = fc;
-                else *reinterpret_cast<bf16x8*>(sFCw + r * LDC + (ks - KCR) * 16 + half * 8) = fc.v;     // read back by the same lane only
             }
         }
         for (int64_t hh = 0; hh < a.hps; ++hh) {
@@ -188,24 +182,6 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                 return lane_xor_add<32>(s);
             };
 
-            // ---- dl_c[i] = e^{l_i} sum_p dy[i][p] (sum_n C[i][n] S_prev[p][n])
-            {
-                floatx16 yo[1][BN];
-                acc_zero(yo);
-#pragma unroll
-                for (int ks = 0; ks < KSN; ++ks) {
-#pragma unroll
-                    for (int j = 0; j < BN; ++j) {
-                        const int row = j * 32 + r;
-                        const Frag<T> bf = load_frag(cP + (row * SPR_S + ((ks * 2 + half) ^ tile_swz<SPR_S>(row))) * 8);
-                        mma_frag(yo[0][j], bf, ks < KCR ? foC[ks < KCR ? ks : 0] : load_frag(sFCw + r * LDC + (ks - KCR) * 16 + half * 8));
-                    }
-                }
-                const float tot = row_dot(yo, cY);
-                if (half == 0) a.dlc[bhc * kQ + tok] = tok < valid ? tot * __expf(sl[tok]) : 0.f;
-            }
-
-            __builtin_amdgcn_sched_barrier(0);
             // ---- state part of dxd: dS (LDS, natural layout) x B rows (registers)
             floatx16 acc[1][BN];
             acc_zero(acc);
@@ -304,41 +280,53 @@ ssd_bwd16_kernel(const Bwd16Args a) {
             if (lane == 0) { a.dDp8[bhc * 8 + wave] = dD_loc; a.dDp8[bhc * 8 + wave + 4] = 0.f; }
         }
     } else {
-        // =============================================================== role B: state parts of dB and dC
+        // =============================================================== role B: state parts of dB and dC, and dl_c
+        // Operands swapped here too: lane (r, half) owns token row0 + r and, per 32-column block jn, the state columns
+        // 32 jn + 8 q + 4 half + 0..3, so the row scales are two scalars per lane.
         floatx16 accB[1][NBN], accC[1][NBN];
         acc_zero(accB);
         acc_zero(accC);
+        const int tok = row0 + r;
+        // C row of this lane's token in accumulator order (the same for every head of the group)
+        uint32_t cw[JCR][4][2];
+        uint2* sCw = sCw_all + rbk * (JCL * 4 * 64);                 // written and read back by the same lane only
+        {
+            const T* Cp = static_cast<const T*>(a.Cm) + b * a.C_sb + (t0 + tok) * a.C_sl + g * a.C_sg;
+#pragma unroll
+            for (int jn = 0; jn < NBN; ++jn)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    uint2 v = uint2{0u, 0u};
+                    if (tok < valid) v = *reinterpret_cast<const uint2*>(Cp + jn * 32 + 8 * q + 4 * half);
+                    if (jn < JCR) { cw[jn < JCR ? jn : 0][q][0] = v.x; cw[jn < JCR ? jn : 0][q][1] = v.y; }
+                    else sCw[((jn - JCR) * 4 + q) * 64 + lane] = v;
+                }
+        }
         for (int64_t hh = 0; hh < a.hps; ++hh) {
             const int64_t h = h_first + hh;
             const int buf = (int)(hh & 1);
             wait_vmem_all();
             const float* sl = sLD + buf * 2 * kQ;
             const float* sd = sl + kQ;
-            // row scales of this wave's 32 tokens, one exponential per token: dt_j e^{Lam - l_j} (dB side, lanes 0-31) and
-            // e^{l_i} (dC side, lanes 32-63; 0 past the end of the sequence)
-            float* wsw = wsB_all + rbk * 64;
-            {
-                const int row = row0 + r;
-                const float lr = sl[row];
-                wsw[lane] = half == 0 ? sd[row] * __expf(sl[kQ - 1] - lr) : (row < valid ? __expf(lr) : 0.f);
-            }
             __syncthreads();
             if (hh + 1 < a.hps) issue_tiles(h + 1, buf ^ 1);
+            // lane-dependent LDS offsets are rebuilt from the lane number for every head (a few integer instructions):
+            // carried across the head loop they are spilled, and every reload waits for the tile copies in flight
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            const int r = ln & 31, half = ln >> 5, tok = row0 + r;
+            const int tr_row = (ln >> 2) & 3, tr_col = ((ln >> 4) & 1) * 16 + 4 * (ln & 3);
+            // row scales of this lane's token: dt_j e^{Lam - l_j} (dB side) and e^{l_i} (dC side and dl_c; 0 past the end)
+            const float lr = sl[tok];
+            const float ws_b = sd[tok] * __expf(sl[kQ - 1] - lr);
+            const float ws_c = tok < valid ? __expf(lr) : 0.f;
             const T* cS = tiles + buf * TILES;
             const T* cP = cS + P * N;
             const T* cY = cP + P * N;
             const T* cX = cY + kQ * P;
-            const int tok = row0 + r;
-            // t[n-block] = sum_p Rows[tok][p] * St[p][n]: rows as they lie (A operand), the state tile through transpose reads
-            auto rows_times_state = [&](const T* Rows, const T* St, bool side_b, floatx16 (&accum)[1][NBN]) {
-                // row scales of this lane's 16 accumulator rows (rows 8 q + 4 half + 0..3: four consecutive table entries)
-                float ws[16];
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const floatx4 w4 = *reinterpret_cast<const floatx4*>(wsw + (side_b ? 0 : 32) + 8 * q + 4 * half);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) ws[4 * q + e] = w4[e];
-                }
+            float dlc = 0.f;
+            // t[tok][n] = sum_p Rows[tok][p] * St[p][n]: the state tile through transpose reads, the rows as they lie
+            auto rows_times_state = [&](const T* Rows, const T* St, const float ws, bool with_c, floatx16 (&accum)[1][NBN]) {
 #pragma unroll
                 for (int jn = 0; jn < NBN; ++jn) {
                     floatx16 t = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -353,24 +341,38 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                         Frag<T> bf;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) { bf.v[e] = lo[e]; bf.v[4 + e] = hi[e]; }
-                        mma_frag(t, load_frag(Rows + (tok * SPR_X + ((ks * 2 + half) ^ tile_swz<SPR_X>(tok))) * 8), bf);
+                        mma_frag(t, bf, load_frag(Rows + (tok * SPR_X + ((ks * 2 + half) ^ tile_swz<SPR_X>(tok))) * 8));
                     }
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) accum[0][jn][v] += t[v] * ws[v];
+                    for (int v = 0; v < 16; ++v) accum[0][jn][v] += t[v] * ws;
+                    asm volatile("" : "+v"(accum[0][jn]));      // the scaled sum is formed here, not after the last block
+                    if (with_c) {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            uint2 cv;
+                            if (jn < JCR) cv = uint2{cw[jn < JCR ? jn : 0][q][0], cw[jn < JCR ? jn : 0][q][1]};
+                            else cv = sCw[((jn - JCR) * 4 + q) * 64 + ln];
+                            dlc += t[4 * q + 0] * unpack_lo<T>(cv.x) + t[4 * q + 1] * unpack_hi<T>(cv.x) +
+                                   t[4 * q + 2] * unpack_lo<T>(cv.y) + t[4 * q + 3] * unpack_hi<T>(cv.y);
+                        }
+                    }
                     __builtin_amdgcn_sched_barrier(0);      // keep the next block's operand reads from being hoisted up here
                 }
             };
-            rows_times_state(cX, cS, true, accB);
-            rows_times_state(cY, cP, false, accC);
+            rows_times_state(cX, cS, ws_b, false, accB);
+            rows_times_state(cY, cP, ws_c, true, accC);
+            // dl_c[i] = e^{l_i} sum_n C[i][n] (sum_p dy[i][p] S_prev[p][n])
+            dlc = lane_xor_add<32>(dlc);
+            if (half == 0) a.dlc[((b * a.nheads + h) * a.nchunks + c) * kQ + tok] = dlc * ws_c;
         }
-        const int64_t part = (((b * a.nchunks + c) * a.ngroups + g) * a.nslices + slice) * (int64_t)(kQ * N);
+        const int64_t part = (((b * a.nchunks + c) * a.ngroups + g) * a.nslices + slice) * (int64_t)(kQ * N) + (int64_t)tok * N;
 #pragma unroll
         for (int jn = 0; jn < NBN; ++jn)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int64_t o = part + (row0 + acc_row(lane, v)) * N + jn * 32 + r;
-                a.dBp[o] = accB[0][jn][v];
-                a.dCp[o] = accC[0][jn][v];
+            for (int q = 0; q < 4; ++q) {
+                const int64_t o = part + jn * 32 + 8 * q + 4 * half;
+                *reinterpret_cast<floatx4*>(a.dBp + o) = floatx4{accB[0][jn][4 * q], accB[0][jn][4 * q + 1], accB[0][jn][4 * q + 2], accB[0][jn][4 * q + 3]};
+                *reinterpret_cast<floatx4*>(a.dCp + o) = floatx4{accC[0][jn][4 * q], accC[0][jn][4 * q + 1], accC[0][jn][4 * q + 2], accC[0][jn][4 * q + 3]};
             }
     }
 }
