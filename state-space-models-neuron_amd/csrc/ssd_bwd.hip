@@ -510,7 +510,8 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
     if (!p->chunk_states && (rc = ssd_launch_states<T, P, N>(p, w, nullptr, st))) return rc;
     // gradient of the state leaving each chunk (reverse recurrence over the chunks' own contributions)
     if constexpr (sizeof(T) == 2) {
-        auto k = state_pass16_kernel<T, P, N, true>;
+        // the main backward kernel forms dlam itself when it runs; otherwise this pass does (and reads the forward states for it)
+        auto k = state_pass16_kernel<T, P, N, true, !bwd16_ok<T, P, N>()>;
         const size_t sm = state_pass_smem<P, N>();
         if ((rc = allow_smem(k, sm))) return rc;
         StatePassArgs sa;
@@ -599,7 +600,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
             m.dy = p->dy; m.dy_sb = p->dy_stride_b; m.dy_sl = p->dy_stride_l; m.dy_sh = p->dy_stride_h;
             m.x = p->x; m.x_sb = p->x_stride_b; m.x_sl = p->x_stride_l; m.x_sh = p->x_stride_h;
             m.dx = p->dx; m.dx_sb = p->dx_stride_b; m.dx_sl = p->dx_stride_l; m.dx_sh = p->dx_stride_h;
-            m.dirp = w.dirp; m.rbp = w.rbp; m.dlc = w.dlc; m.dDp8 = w.dDp8; m.dBp = w.dBp; m.dCp = w.dCp;
+            m.dirp = w.dirp; m.rbp = w.rbp; m.dlc = w.dlc; m.dDp8 = w.dDp8; m.dlam = w.dlam; m.dBp = w.dBp; m.dCp = w.dCp;
             m.seqlen = p->seqlen; m.nheads = p->nheads; m.ngroups = p->ngroups; m.nchunks = nc;
             m.nslices = w.ns_b; m.hps = w.hps_b;
             auto k = ssd_bwd16_kernel<T, P, N>;

@@ -19,6 +19,8 @@
 // Every MFMA is issued with its operands swapped, so a lane's accumulators belong to ONE token: row scales and row dot
 // products are lane-local (plus one exchange with the partner lane), and dx leaves in 16-byte stores after one
 // lane-pair swap per 4-channel group, without a pass through LDS.
+// All eight waves also form   dlam[c] = e^{Lam_c} <dS, S_prev>   (the part of dL/dLam_c that flows through the carried
+// state) from the two tiles as they lie in LDS, one partial per wave.
 // The decay is factorised per row block around its LAST token (see ssd_diag.hpp), with the exact per-element
 // fallback when the block's range exceeds kMaxRange.  ddt and dA need a scan over the chunk and are left to da_body (tail1_kernel).
 #pragma once
@@ -48,6 +50,7 @@ struct Bwd16Args {
     void* dx; int64_t dx_sb, dx_sl, dx_sh;
     float* dirp; float* rbp; float* dlc;                  // [b][h][c][kQ]
     float* dDp8;                                          // [b][h][c][8]
+    float* dlam;                                          // [b][h][c][kDlamParts]
     float* dBp; float* dCp;                               // [b][c][g][slice][kQ][N]
     int64_t seqlen, nheads, ngroups, nchunks, nslices, hps;
 };
@@ -57,6 +60,7 @@ __global__ void __launch_bounds__(512, 1)
 ssd_bwd16_kernel(const Bwd16Args a) {
     static_assert(sizeof(T) == 2, "16-bit operands only");
     constexpr int BN = P / 32, KSN = N / 16, KSP = P / 16, NBN = N / 32;
+    static_assert(kDlamParts == 8 && (P * N) % (512 * 8) == 0, "one dlam partial per wave");
     constexpr int SPR_S = N / 8, SPR_X = P / 8;
     constexpr int NS = P * SPR_S / 512, NX = kQ * SPR_X / 512;
     constexpr int TAB = kQ + 32;
@@ -115,6 +119,24 @@ ssd_bwd16_kernel(const Bwd16Args a) {
         }
         async_copy_ldtab(a.ldtab, (b * a.nheads + h) * a.nchunks + c, lds_LD + (uint32_t)(buf * 2 * kQ * 4));
     };
+    // this wave's share of <dS, S_prev> over the two tiles of buffer `buf` (same slot order in both, so any order will do)
+    auto tiles_dot = [&](int buf, int64_t bhc, float Lam) {
+        const T* cS = tiles + buf * TILES;
+        const T* cP = cS + P * N;
+        int t = tid;
+        asm volatile("" : "+v"(t));
+        float dot = 0.f;
+#pragma unroll
+        for (int it = 0; it < P * N / (512 * 8); ++it) {
+            const uint4 u = *reinterpret_cast<const uint4*>(cS + (it * 512 + t) * 8);
+            const uint4 v = *reinterpret_cast<const uint4*>(cP + (it * 512 + t) * 8);
+            const uint32_t uw[4] = {u.x, u.y, u.z, u.w}, vw[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) dot += unpack_lo<T>(uw[q]) * unpack_lo<T>(vw[q]) + unpack_hi<T>(uw[q]) * unpack_hi<T>(vw[q]);
+        }
+        dot = warp_sum(dot);
+        if (lane == 0) a.dlam[bhc * kDlamParts + wave] = __expf(Lam) * dot;
+    };
     issue_tiles(h_first, 0);
 
     if (role == 0) {
@@ -155,6 +177,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
             if (lane < 32) wu[lane] = __expf(fminf(lref - sl[row0 + lane], 0.f));
             __syncthreads();
             if (hh + 1 < a.hps) issue_tiles(h + 1, buf ^ 1);
+            tiles_dot(buf, bhc, Lam);
             const T* cS = tiles + buf * TILES;
             const T* cP = cS + P * N;
             const T* cY = cP + P * N;
@@ -316,6 +339,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
             asm volatile("" : "+v"(ln));
             const int r = ln & 31, half = ln >> 5, tok = row0 + r;
             const int tr_row = (ln >> 2) & 3, tr_col = ((ln >> 4) & 1) * 16 + 4 * (ln & 3);
+            tiles_dot(buf, (b * a.nheads + h) * a.nchunks + c, sl[kQ - 1]);
             // row scales of this lane's token: dt_j e^{Lam - l_j} (dB side) and e^{l_i} (dC side and dl_c; 0 past the end)
             const float lr = sl[tok];
             const float ws_b = sd[tok] * __expf(sl[kQ - 1] - lr);
@@ -327,6 +351,9 @@ ssd_bwd16_kernel(const Bwd16Args a) {
             float dlc = 0.f;
             // t[tok][n] = sum_p Rows[tok][p] * St[p][n]: the state tile through transpose reads, the rows as they lie
             auto rows_times_state = [&](const T* Rows, const T* St, const float ws, bool with_c, floatx16 (&accum)[1][NBN]) {
+                Frag<T> af[KSP];
+#pragma unroll
+                for (int ks = 0; ks < KSP; ++ks) af[ks] = load_frag(Rows + (tok * SPR_X + ((ks * 2 + half) ^ tile_swz<SPR_X>(tok))) * 8);
 #pragma unroll
                 for (int jn = 0; jn < NBN; ++jn) {
                     floatx16 t = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -341,7 +368,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                         Frag<T> bf;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) { bf.v[e] = lo[e]; bf.v[4 + e] = hi[e]; }
-                        mma_frag(t, bf, load_frag(Rows + (tok * SPR_X + ((ks * 2 + half) ^ tile_swz<SPR_X>(tok))) * 8));
+                        mma_frag(t, bf, af[ks]);
                     }
 #pragma unroll
                     for (int v = 0; v < 16; ++v) accum[0][jn][v] += t[v] * ws;

@@ -4,7 +4,9 @@
 //   forward:  S = init;   for c = 0 .. nc-1:   prev[c] = T(S);   S = e^{Lam_c} S + sum_j (dt_j e^{Lam_c - l_j}) x_j (x) B_j;   final = S
 //   reverse:  R = dfinal; for c = nc-1 .. 0:   prev[c] = T(R);   dlam[c] = e^{Lam_c} <T(R), sprev[c]>;
 //                                              R = e^{Lam_c} R + sum_i e^{l_i} dy_i (x) C_i;   dinit = R
-// (dlam is the part of dL/dLam_c that flows through the carried state; sprev[c] = the forward state entering chunk c.)
+// (dlam is the part of dL/dLam_c that flows through the carried state; sprev[c] = the forward state entering chunk c.
+//  With DLAM == false the reverse pass leaves dlam to ssd_bwd16_kernel, which has both tiles in LDS anyway, and does
+//  not read sprev at all.)
 //
 // grid (nheads * NSPLIT, batch), 2 x NWG waves; a workgroup owns N / NSPLIT columns of the [P][N] state, wave w rows
 // [ (w & 1) P/2, +P/2 ) x one NWG-th of those columns, as 32x32 MFMA accumulator blocks.  Per chunk the MFMA computes  X_scaled^T [P x kQ] * M [kQ x N]:
@@ -49,8 +51,8 @@ constexpr size_t state_pass_smem() {
     return (size_t)2 * kQ * P * 2 + (size_t)2 * state_pass_nwg<N>() * (P / 2) * (N / state_pass_nsplit<N>() / state_pass_nwg<N>() + 8) * 2;
 }
 
-template <typename T, int P, int N, bool REVERSE>
-__global__ void __launch_bounds__(state_pass_threads<N>(), (P == 64 ? (REVERSE ? 2 : 3) : (REVERSE ? 1 : 2)))
+template <typename T, int P, int N, bool REVERSE, bool DLAM = REVERSE>
+__global__ void __launch_bounds__(state_pass_threads<N>(), (P == 64 ? (DLAM ? 2 : 3) : (DLAM ? 1 : 2)))
 state_pass16_kernel(const StatePassArgs a) {
     static_assert(sizeof(T) == 2, "16-bit operands only");
     constexpr int NSPLIT = state_pass_nsplit<N>();
@@ -129,7 +131,8 @@ state_pass16_kernel(const StatePassArgs a) {
     // exactly and leaves the next chunk's rows, issued behind them, in flight): the group's B^T / C^T fragments (L2) and,
     // for the reverse pass, this lane's pieces of the forward state
     Frag<T> bf[NBW][8];
-    u32x4 spr[REVERSE ? NSP : 1];
+    static_assert(REVERSE || !DLAM, "dlam belongs to the reverse pass");
+    u32x4 spr[DLAM ? NSP : 1];
     const uint32_t st_off = (uint32_t)(((pw * (P / 2) + lane / LPR) * N + n0 + (lane % LPR) * 8) * 2);      // pass ps: + ps * RPP * N * 2
     auto load_same = [&](int64_t c) {
         const char* mp = reinterpret_cast<const char*>(static_cast<const T*>(a.Mt) + ((b * nc + c) * a.ngroups + g) * (int64_t)(N * kQ));
@@ -138,7 +141,7 @@ state_pass16_kernel(const StatePassArgs a) {
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks)      // see mt_offset
                 bf[j][ks].v = *reinterpret_cast<const bf16x8*>(mp + ((uint32_t)lane * 16u + (uint32_t)((((n0 >> 5) + j) * 8 + ks) * 1024)));
-        if (REVERSE) {
+        if (DLAM) {
             const char* sp = reinterpret_cast<const char*>(static_cast<const T*>(a.sprev) + ((b * nc + c) * a.nheads + h) * (int64_t)(P * N));
 #pragma unroll
             for (int ps = 0; ps < NSP; ++ps) spr[ps] = *reinterpret_cast<const u32x4*>(sp + (st_off + (uint32_t)(ps * RPP * N * 2)));
@@ -191,13 +194,13 @@ state_pass16_kernel(const StatePassArgs a) {
             const int rl = ps * RPP + lane / LPR, cv = lane % LPR;
             const u32x4 o = *reinterpret_cast<const u32x4*>(sOw + rl * LDO + cv * 8);
             *reinterpret_cast<u32x4*>(op + (st_off + (uint32_t)(ps * RPP * N * 2))) = o;
-            if (REVERSE) {
+            if (DLAM) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
                     dot += unpack_lo<T>(o[q]) * unpack_lo<T>(spr[ps][q]) + unpack_hi<T>(o[q]) * unpack_hi<T>(spr[ps][q]);
             }
         }
-        if (REVERSE) {
+        if (DLAM) {
             dot = warp_sum(dot);
             if (lane == 0) {
                 const int slot = (int)(blockIdx.x / a.nheads) * (2 * NWG) + wave;
