@@ -140,6 +140,8 @@ ssd_bwd16_kernel(const Bwd16Args a) {
     issue_tiles(h_first, 0);
 
     if (role == 0) {
+        // role A is the longer of the two: its waves go first whenever both waves of a SIMD are ready
+        __builtin_amdgcn_s_setprio(2);
         // =============================================================== role A: dx, dir, rb, dl_c, dD
         float* wv = wt_all + rbk * TAB;
         float* wu = wv + kQ;

@@ -151,6 +151,15 @@ state_pass16_kernel(const StatePassArgs a) {
     auto step = [&](int64_t cc, Ahead& s) {
         const int64_t c = chunk_of(cc);
         const int buf = (int)(cc & 1);
+        // Issue priority falls as the workgroup advances, so that of the workgroups sharing a CU the one furthest behind
+        // goes first: the hardware otherwise prefers the oldest waves, and the last workgroup placed on a CU that holds
+        // one more than its neighbours finishes long after everybody else.
+        switch ((int)(cc * 4 / nc)) {
+            case 0: __builtin_amdgcn_s_setprio(3); break;
+            case 1: __builtin_amdgcn_s_setprio(2); break;
+            case 2: __builtin_amdgcn_s_setprio(1); break;
+            default: __builtin_amdgcn_s_setprio(0); break;
+        }
         T* cX = sX + buf * (kQ * P);
         __builtin_amdgcn_sched_barrier(0);      // keep this chunk's loads out of the previous chunk's MFMA phase (registers)
         load_same(c);
