@@ -152,7 +152,7 @@ inline int allow_smem(K kernel, size_t bytes) {
 template <typename T, int P, int N>
 inline size_t state_smem() { return (size_t)(P + N) * lds_ld<T>(kQ) * sizeof(T); }
 template <typename T>
-inline size_t cb_smem(int n) { return (size_t)2 * kQ * lds_ld<T>(n) * sizeof(T); }
+inline size_t cb_smem(int n) { return (size_t)2 * 64 * lds_ld<T>(n) * sizeof(T); }
 
 // Decay tables, G = C B^T (+ operand tiles), local chunk states, forward state scan.  Used by the forward and, when the
 // caller did not keep the forward's chunk_states buffer, by the backward (recompute).
@@ -178,7 +178,7 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
         pa.seqlen = p->seqlen; pa.nheads = p->nheads; pa.ngroups = p->ngroups; pa.nchunks = nc;
         pa.total_bhc = p->batch * p->nheads * nc;
         pa.n_cb = nc * p->ngroups * p->batch;
-        const int64_t blocks = 2 * pa.n_cb + ceil_div(pa.total_bhc, (int64_t)4);
+        const int64_t blocks = kCbParts * pa.n_cb + ceil_div(pa.total_bhc, (int64_t)4);
         M2_REQUIRE(blocks < ((int64_t)1 << 31), M2_ERR_SHAPE, "ssd: too many workgroups");
         k<<<(unsigned)blocks, 256, sm, st>>>(pa);
         if ((rc = check_launch("ssd prep_kernel"))) return rc;

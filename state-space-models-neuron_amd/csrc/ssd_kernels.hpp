@@ -32,9 +32,8 @@ namespace m2 {
 //   Gmt [kQ][kQ] T               its transpose: Gmt[j][i] = G[i][j] for i >= j (backward dx term, rows j)
 //   Bt, Ct N x kQ T              B and C transposed (tokens contiguous), laid out by mt_offset: MFMA operands of the
 //                                chunk-state products
-// Two workgroups of 256 threads per (chunk, group, batch): one for G and its two operand-type copies, one for the
-// transposed tiles (independent work on the same inputs).  The upper-right 64x64 quadrant of G is never consumed and
-// is neither computed nor written.
+// kCbParts workgroups of 256 threads per (chunk, group, batch), see cb_body.  The upper-right 64x64 quadrant of G is
+// never consumed and is neither computed nor written.
 // Element offset of the 8 tokens s0 .. s0 + 7 (s0 a multiple of 8) of state column n inside a transposed B / C tile.
 //   fp32   : [N][kQ], tokens contiguous (rows staged into LDS by chunk_state_kernel);
 //   16-bit : MFMA operand order [N / 32][kQ / 16][64 lanes][8]: the B-operand fragment of a wave for column block n / 32
@@ -46,72 +45,74 @@ __device__ __forceinline__ int64_t mt_offset(int n, int s0) {
     return (int64_t)n * kQ + s0;
 }
 
+// Workgroups per (chunk, group, batch): three for the 64x64 quadrants of G on and below the diagonal, four for the
+// transposed tiles (32 tokens each) -- seven short independent pieces rather than two long ones.
+constexpr int kCbParts = 7;
 template <typename T, int N>
 __device__ __forceinline__ void
 cb_body(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict__ Gf, T* __restrict__ Gm, T* __restrict__ Gmt,
         T* __restrict__ Bt, T* __restrict__ Ct,
         int64_t seqlen, int64_t ngroups, int64_t nchunks,
         int64_t Bsb, int64_t Bsl, int64_t Bsg, int64_t Csb, int64_t Csl, int64_t Csg, int64_t c, int64_t g, int64_t b,
-        const bool transposes) {
-    constexpr int KB = N;          // the whole contraction length at once: one staging phase, one barrier pair
-    constexpr int LD = lds_ld<T>(KB);
+        const int part) {
+    constexpr int LD = lds_ld<T>(N);      // the whole contraction length at once: one staging phase, one barrier
     constexpr int V = VecTraits<T>::kVec;
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    T* sC = reinterpret_cast<T*>(smem_raw);
-    T* sB = sC + kQ * LD;
+    T* sC = reinterpret_cast<T*>(smem_raw);      // [64][LD]
+    T* sB = sC + 64 * LD;                        // [64][LD]
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int64_t t0 = c * kQ;
     const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
     const T* Bp = Bm + b * Bsb + t0 * Bsl + g * Bsg;
     const T* Cp = Cm + b * Csb + t0 * Csl + g * Csg;
     const int64_t grp = (b * nchunks + c) * ngroups + g;
-    T* Btp = Bt + grp * (int64_t)(N * kQ);
-    T* Ctp = Ct + grp * (int64_t)(N * kQ);
-    const int wm = wave >> 1, wn = wave & 1;
-    floatx16 acc[2][2];
-    acc_zero(acc);
-    for (int k0 = 0; k0 < N; k0 += KB) {
-        stage_rows<T, kQ, KB, 256, false>(sC, LD, Cp + k0, Csl, valid, nullptr, tid);
-        stage_rows<T, kQ, KB, 256, false>(sB, LD, Bp + k0, Bsl, valid, nullptr, tid);
+    if (part >= 3) {
+        // transposed copies of tokens [tk0, tk0 + 32): thread -> (state column n, group of V tokens)
+        const int tk0 = (part - 3) * 32;
+        T* Btp = Bt + grp * (int64_t)(N * kQ);
+        T* Ctp = Ct + grp * (int64_t)(N * kQ);
+        stage_rows<T, 32, N, 256, false>(sC, LD, Cp + (int64_t)tk0 * Csl, Csl, valid - tk0, nullptr, tid);
+        stage_rows<T, 32, N, 256, false>(sB, LD, Bp + (int64_t)tk0 * Bsl, Bsl, valid - tk0, nullptr, tid);
         __syncthreads();
-        if (!transposes && !(wm == 0 && wn == 1)) wave_mma<2, 2>(acc, sC + wm * 64 * LD, LD, sB + wn * 64 * LD, LD, 0, KB);
-        // transposed copies of this 64-column slab: thread -> (state column n, group of V tokens)
-        for (int e = tid; transposes && e < KB * (kQ / V); e += 256) {
-            const int n = e % KB, s0 = (e / KB) * V;
+        for (int e = tid; e < N * (32 / V); e += 256) {
+            const int n = e % N, s0 = (e / N) * V;
             T vb[V], vc[V];
 #pragma unroll
             for (int q = 0; q < V; ++q) { vb[q] = sB[(s0 + q) * LD + n]; vc[q] = sC[(s0 + q) * LD + n]; }
-            *reinterpret_cast<uint4*>(Btp + mt_offset<T>(k0 + n, s0)) = *reinterpret_cast<const uint4*>(vb);
-            *reinterpret_cast<uint4*>(Ctp + mt_offset<T>(k0 + n, s0)) = *reinterpret_cast<const uint4*>(vc);
+            *reinterpret_cast<uint4*>(Btp + mt_offset<T>(n, tk0 + s0)) = *reinterpret_cast<const uint4*>(vb);
+            *reinterpret_cast<uint4*>(Ctp + mt_offset<T>(n, tk0 + s0)) = *reinterpret_cast<const uint4*>(vc);
         }
-        __syncthreads();
+        return;
     }
-    if (transposes || (wm == 0 && wn == 1)) return;
+    // quadrant (wm, wn) of G = C B^T; wave (wi, wj) takes one 32x32 block of it
+    const int wm = part == 0 ? 0 : 1, wn = part == 2 ? 1 : 0;
+    const int wi = wave >> 1, wj = wave & 1;
+    stage_rows<T, 64, N, 256, false>(sC, LD, Cp + (int64_t)(wm * 64) * Csl, Csl, valid - wm * 64, nullptr, tid);
+    stage_rows<T, 64, N, 256, false>(sB, LD, Bp + (int64_t)(wn * 64) * Bsl, Bsl, valid - wn * 64, nullptr, tid);
+    __syncthreads();
+    if (wm * 2 + wi < wn * 2 + wj) return;          // block above the diagonal
+    floatx16 acc[1][1];
+    acc_zero(acc);
+    wave_mma<1, 1>(acc, sC + wi * 32 * LD, LD, sB + wj * 32 * LD, LD, 0, N);
     float* Gfp = Gf + grp * (int64_t)(kQ * kQ);
     T* Gmp = Gm + grp * (int64_t)(kQ * kQ);
     T* Gmtp = Gmt + grp * (int64_t)(kQ * kQ);
+    const int col = wn * 64 + wj * 32 + acc_col(lane);
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int q = 0; q < 4; ++q) {
+        const int rowq = wm * 64 + wi * 32 + 8 * q + 4 * (lane >> 5);
+        T mt[4];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            if (wm * 2 + i < wn * 2 + j) continue;          // block above the diagonal
-            const int col = wn * 64 + j * 32 + acc_col(lane);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int rowq = wm * 64 + i * 32 + 8 * q + 4 * (lane >> 5);
-                T mt[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int row = rowq + e;
-                    const float gv = acc[i][j][4 * q + e];
-                    const float gm = row >= col ? gv : 0.f;
-                    Gfp[row * kQ + col] = gv;
-                    Gmp[row * kQ + col] = from_f32<T>(gm);
-                    mt[e] = from_f32<T>(gm);
-                }
-                *reinterpret_cast<RawVec<T, 4>*>(Gmtp + col * kQ + rowq) = *reinterpret_cast<const RawVec<T, 4>*>(mt);
-            }
+        for (int e = 0; e < 4; ++e) {
+            const int row = rowq + e;
+            const float gv = acc[0][0][4 * q + e];
+            const float gm = row >= col ? gv : 0.f;
+            Gfp[row * kQ + col] = gv;
+            Gmp[row * kQ + col] = from_f32<T>(gm);
+            mt[e] = from_f32<T>(gm);
         }
+        *reinterpret_cast<RawVec<T, 4>*>(Gmtp + col * kQ + rowq) = *reinterpret_cast<const RawVec<T, 4>*>(mt);
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -137,7 +138,7 @@ ld_table_body(const void* __restrict__ dt, int dt_f32, const float* __restrict__
 }
 
 // Both preparations in one launch (they are independent, and either alone leaves most of the GPU idle): the first
-// 2 n_cb workgroups run cb_body for (part, chunk, group, batch) = the index split in that order, the others ld_table_body.
+// kCbParts n_cb workgroups run cb_body for (part, chunk, group, batch) = the index split in that order, the others ld_table_body.
 struct PrepArgs {
     const void* Bm; const void* Cm; float* Gf; void* Gm; void* Gmt; void* Bt; void* Ct;
     int64_t Bsb, Bsl, Bsg, Csb, Csl, Csg;
@@ -148,14 +149,14 @@ template <typename T, int N>
 __global__ void __launch_bounds__(256)
 prep_kernel(const PrepArgs a) {
     const int64_t blk = blockIdx.x;
-    if (blk < 2 * a.n_cb) {
-        const int64_t q = blk >> 1;
+    if (blk < kCbParts * a.n_cb) {
+        const int64_t q = blk / kCbParts;
         const int64_t c = q % a.nchunks, g = (q / a.nchunks) % a.ngroups, b = q / (a.nchunks * a.ngroups);
         cb_body<T, N>(static_cast<const T*>(a.Bm), static_cast<const T*>(a.Cm), a.Gf, static_cast<T*>(a.Gm), static_cast<T*>(a.Gmt),
                       static_cast<T*>(a.Bt), static_cast<T*>(a.Ct), a.seqlen, a.ngroups, a.nchunks,
-                      a.Bsb, a.Bsl, a.Bsg, a.Csb, a.Csl, a.Csg, c, g, b, (blk & 1) != 0);
+                      a.Bsb, a.Bsl, a.Bsg, a.Csb, a.Csl, a.Csg, c, g, b, (int)(blk % kCbParts));
     } else {
-        ld_table_body<T>(a.dt, a.dt_f32, a.A, a.ldtab, a.lam, a.seqlen, a.nheads, a.nchunks, a.total_bhc, a.dtsb, a.dtsl, blk - 2 * a.n_cb);
+        ld_table_body<T>(a.dt, a.dt_f32, a.A, a.ldtab, a.lam, a.seqlen, a.nheads, a.nchunks, a.total_bhc, a.dtsb, a.dtsl, blk - kCbParts * a.n_cb);
     }
 }
 
