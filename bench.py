@@ -27,7 +27,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0     # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0              # MI355X HBM3E
 # Measured HBM bytes per step (rocprofv3 FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, the factors the 1 GiB copy kernel
 # gives in the same runs; profiles/bench_all_workloads_kernels.md).  They describe the kernels as profiled, not this run.
-SSD_TRAFFIC_BYTES = 1.465e9
+SSD_TRAFFIC_BYTES = 1.441e9
 CONV_TRAFFIC_BYTES = 459.5e6
 DECODE_TRAFFIC_BYTES = 64 * 689.3e6
 
