@@ -13,6 +13,8 @@
  *                                         :277-485 (mamba_kernel_bwd_); wrapper :488-519
  *   m2_decode_step                     <- mamba2/mamba2_kernel_inference.py:27-104
  *                                         (mamba_inference_kernel_); wrapper :107-122
+ *   m2_softplus_bias_* / m2_rmsnorm_gated_*  <- mamba2/fused_kernel.py:24-175 (glue kernels of the
+ *                                         fused mixer core)
  *
  * Conventions
  *   - Every pointer is a DEVICE pointer owned by the caller (inputs, outputs and
@@ -149,6 +151,48 @@ typedef struct m2_decode_params {
 
 size_t m2_decode_workspace_bytes(int64_t batch, int64_t nheads, int64_t headdim, int64_t dstate, int64_t ngroups);
 int m2_decode_step(const m2_decode_params* p, void* stream);
+
+/* ------------------------------------------------------------------ mixer glue
+ * The elementwise passes between the conv, the scan and the output projection
+ * (mamba2/fused_kernel.py:24-47 softplus_with_bias, :50-73 softplus_with_bias_bwd,
+ * :76-105 rmsnorm, :128-175 rmsnorm_bwd; torch twins mamba2/mamba2_mixer.py:36-38, 88-105).
+ * Rows are (batch x token) pairs; the channel dimension is contiguous, rows may be strided
+ * (columns of the packed [z | xBC | dt] projection output and of its gradient).
+ *
+ * softplus:  out = softplus(dt + dt_bias[h]) in the threshold form (x for x >= 10);
+ *            d_in = d_out * sigmoid(dt + dt_bias) (1 above the threshold), d_bias[h] = sum over rows, fp32.
+ * rmsnorm:   h = x * silu(z) (h = x without z);  out = weight * h * rsqrt(mean(h^2) + eps) with the mean
+ *            taken inside each of n_groups groups of channels / n_groups contiguous channels.
+ *            Backward: dx, dz (same type as x) and d_weight (fp32, summed over the rows).
+ *            Channels per group: a multiple of 8 (bf16) / 4 (fp32), at most 8192 (bf16) / 4096 (fp32).
+ * dt_bias, weight, d_bias, d_weight are fp32.  The backward entry points take a workspace of
+ * m2_*_bwd_workspace_bytes() bytes (per-block partial sums, added in a fixed order: no atomics).
+ */
+int m2_softplus_bias_fwd(const void* dt, int64_t dt_stride_row, const float* dt_bias, void* out, int64_t out_stride_row,
+                         int64_t rows, int64_t nheads, int32_t dtype, void* stream);
+size_t m2_softplus_bias_bwd_workspace_bytes(int64_t rows, int64_t nheads);
+int m2_softplus_bias_bwd(const void* dt, int64_t dt_stride_row, const float* dt_bias, const void* d_out, int64_t d_out_stride_row,
+                         void* d_in, int64_t d_in_stride_row, float* d_bias, void* workspace, size_t workspace_bytes,
+                         int64_t rows, int64_t nheads, int32_t dtype, void* stream);
+
+typedef struct m2_rmsnorm_params {
+    const void* x; const void* z;                       /* (rows, channels); z may be NULL (no gate)   */
+    const float* weight;                                /* (channels)                                   */
+    void* out;                                          /* forward: (rows, channels)                    */
+    const void* d_out; void* dx; void* dz;              /* backward; dz required when z is given        */
+    float* d_weight;                                    /* backward: (channels) fp32                    */
+    void* workspace; size_t workspace_bytes;            /* backward only                                */
+    int64_t rows, channels;
+    int64_t x_stride_row, z_stride_row, out_stride_row, d_out_stride_row, dx_stride_row, dz_stride_row;
+    int32_t n_groups;
+    int32_t dtype;                                      /* x, z, d_out, dx, dz (and out unless out_f32) */
+    int32_t out_f32;                                    /* forward output in fp32 (mamba2_mixer.py:104-105) */
+    float eps;
+} m2_rmsnorm_params;
+
+int m2_rmsnorm_gated_fwd(const m2_rmsnorm_params* p, void* stream);
+size_t m2_rmsnorm_gated_bwd_workspace_bytes(int64_t rows, int64_t channels, int32_t n_groups, int32_t dtype);
+int m2_rmsnorm_gated_bwd(const m2_rmsnorm_params* p, void* stream);
 
 /* ------------------------------------------------------------------ self tests / probes
  * m2_mfma_selftest: C (M x N fp32, row-major) = A (M x K) * Bt (N x K)^T through the same

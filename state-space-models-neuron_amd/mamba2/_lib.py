@@ -59,6 +59,15 @@ class DecodeParams(C.Structure):
                 ("dtype", _i32), ("param_dtype", _i32), ("activation", _i32)]
 
 
+class RmsnormParams(C.Structure):
+    _fields_ = [("x", _vp), ("z", _vp), ("weight", _vp), ("out", _vp), ("d_out", _vp), ("dx", _vp), ("dz", _vp), ("d_weight", _vp),
+                ("workspace", _vp), ("workspace_bytes", _sz),
+                ("rows", _i64), ("channels", _i64),
+                ("x_stride_row", _i64), ("z_stride_row", _i64), ("out_stride_row", _i64), ("d_out_stride_row", _i64),
+                ("dx_stride_row", _i64), ("dz_stride_row", _i64),
+                ("n_groups", _i32), ("dtype", _i32), ("out_f32", _i32), ("eps", C.c_float)]
+
+
 # name -> (restype, argtypes); every symbol the header declares
 SYMBOLS = {
     "m2_abi_version": (C.c_int, []),
@@ -73,6 +82,12 @@ SYMBOLS = {
     "m2_ssd_bwd": (C.c_int, [C.POINTER(SsdParams), _vp]),
     "m2_decode_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64]),
     "m2_decode_step": (C.c_int, [C.POINTER(DecodeParams), _vp]),
+    "m2_softplus_bias_fwd": (C.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _i64, _i32, _vp]),
+    "m2_softplus_bias_bwd_workspace_bytes": (_sz, [_i64, _i64]),
+    "m2_softplus_bias_bwd": (C.c_int, [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _sz, _i64, _i64, _i32, _vp]),
+    "m2_rmsnorm_gated_fwd": (C.c_int, [C.POINTER(RmsnormParams), _vp]),
+    "m2_rmsnorm_gated_bwd_workspace_bytes": (_sz, [_i64, _i64, _i32, _i32]),
+    "m2_rmsnorm_gated_bwd": (C.c_int, [C.POINTER(RmsnormParams), _vp]),
     "m2_mfma_selftest": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp]),
     "m2_stream_copy": (C.c_int, [_vp, _vp, _sz, _vp]),
 }

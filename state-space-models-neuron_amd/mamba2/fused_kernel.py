@@ -6,7 +6,7 @@
 Pipeline (``fused_kernel.py:252-282``): split [z | xBC | dt] -> depthwise conv + SiLU ->
 softplus(dt + dt_bias) -> SSD scan -> gated RMSNorm per group (eps 1e-5).
 
-The split is never materialised: the HIP kernels take strided views of ``zxBCdt`` (the conv reads
+Every stage is a HIP kernel.  The split is never materialised: the kernels take strided views of ``zxBCdt`` (the conv reads
 the xBC columns in place; the scan reads x, B, C as views of the conv output), and in the backward
 the scan writes dx, dB, dC straight into one packed buffer and the conv writes its dx straight into
 the xBC columns of ``d_zxBCdt``.  ``Mamba2FusedKernel`` saves only its inputs and recomputes conv,
@@ -48,13 +48,13 @@ def _forward_parts(zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, n_groups, d
     b, l, _ = zxBCdt.shape
     conv_out = torch.empty((b, l, d_conv), dtype=zxBCdt.dtype, device=zxBCdt.device)
     conv1d_forward(xBC, conv_w, conv_b, "silu", channels_last=True, out=conv_out)
-    dt_sp = glue.softplus_bias(dt, dt_bias)
+    dt_sp = glue.softplus_bias_hip(dt, dt_bias)
     x, Bm, Cm = _xbc_views(conv_out, n_groups, d_state, d_inner, d_head)
     # the scan's chunk states are kept for the backward when one follows directly (no second recompute there)
     states = alloc_chunk_states(dt_sp, logA, x, Bm, Cm) if (keep_states and x.numel() > 0) else None
     y, _ = ssd_forward(dt_sp, logA, x, Bm, Cm, D, chunk_states=states)
     scan_out = y.view(b, l, d_inner)
-    norm_out = glue.rmsnorm_gated(scan_out, z, norm_w, n_groups, NORM_EPS, out_dtype=zxBCdt.dtype)
+    norm_out = glue.rmsnorm_gated_hip(scan_out, z, norm_w, n_groups, NORM_EPS, out_dtype=zxBCdt.dtype)
     return norm_out, conv_out, dt_sp, scan_out, states
 
 
@@ -67,7 +67,7 @@ def _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, 
     dxBC_view = d_zxBCdt[..., d_inner:d_inner + d_conv]
     ddt_view = d_zxBCdt[..., d_inner + d_conv:]
     # gated RMSNorm backward: d_scan_out, d_z (written into d_zxBCdt), d_norm_weight
-    d_scan_out, d_norm_w = glue.rmsnorm_gated_bwd(scan_out, z, norm_w, d_output, n_groups, NORM_EPS, out_dz=dz_view)
+    d_scan_out, d_norm_w, _ = glue.rmsnorm_gated_bwd_hip(scan_out, z, norm_w, d_output, n_groups, NORM_EPS, out_dz=dz_view)
     # SSD backward, gradients of x, B, C written into one packed [dx | dB | dC] buffer
     x, Bm, Cm = _xbc_views(conv_out, n_groups, d_state, d_inner, d_head)
     d_conv_out = torch.empty_like(conv_out)
@@ -75,7 +75,7 @@ def _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, 
     d_dt_sp, d_logA, _, _, _, d_D, _ = ssd_backward(dt_sp, logA, x, Bm, Cm, D, d_scan_out.view(b, l, h, d_head),
                                                      out_dX=dx_v, out_dB=dB_v, out_dC=dC_v, chunk_states=states)
     # softplus backward (into the dt columns) and conv backward (into the xBC columns)
-    d_dt_bias = glue.softplus_bias_bwd(dt, dt_bias, d_dt_sp, out_d_in=ddt_view)
+    _, d_dt_bias = glue.softplus_bias_bwd_hip(dt, dt_bias, d_dt_sp, out_d_in=ddt_view)
     _, d_conv_w, d_conv_b = conv1d_backward(xBC, conv_w, conv_b, d_conv_out, "silu", channels_last=True, out_dx=dxBC_view)
     return (d_zxBCdt, d_logA.to(logA.dtype), d_D.to(D.dtype) if D is not None else None, d_conv_w, d_conv_b,
             d_dt_bias.to(dt_bias.dtype), d_norm_w.to(norm_w.dtype))
