@@ -30,6 +30,7 @@ HBM_PEAK_GBS = 8000.0              # MI355X HBM3E
 SSD_TRAFFIC_BYTES = 1.441e9
 CONV_TRAFFIC_BYTES = 459.5e6
 DECODE_TRAFFIC_BYTES = 64 * 689.3e6
+GLUE_TRAFFIC_BYTES = None
 
 SSD_CFG = dict(b=4, l=2048, h=80, p=64, n=128, g=1)
 CONV_CFG = dict(b=4, l=2048, C=5376, k=4)
@@ -108,6 +109,48 @@ def bench_conv(steps, warmup):
                 roofline={"bound": "hbm", "achieved": bytes_ / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": CONV_TRAFFIC_BYTES,
                           "algorithmic_bytes_per_step": bytes_, "kernels": "conv_fwd_cl_kernel + conv_bwd_cl_kernel + conv_reduce_partials_kernel"})
+
+
+def bench_glue(steps, warmup):
+    """Mixer glue at the 2.7B layer shape: gated RMSNorm over d_inner = 5120 (one group) and softplus(dt + bias) over 80
+    heads, forward + backward, with z / dz / dt / ddt as column slices of packed (b, l, 10576) buffers as in the layer."""
+    import torch
+    from mamba2 import glue
+    b, l, d, h, g = SSD_CFG["b"], SSD_CFG["l"], SSD_CFG["h"] * SSD_CFG["p"], SSD_CFG["h"], SSD_CFG["g"]
+    width = 2 * d + 2 * g * SSD_CFG["n"] + h
+    gen = torch.Generator(device="cuda:0").manual_seed(0)
+    nsets = 3          # rotate input sets so the 256 MB MALL does not serve the reads
+    sets = []
+    for _ in range(nsets):
+        packed = torch.randn(b, l, width, device="cuda:0", generator=gen).to(torch.bfloat16)
+        sets.append(dict(packed=packed, x=torch.randn(b, l, d, device="cuda:0", generator=gen).to(torch.bfloat16),
+                         dout=torch.randn(b, l, d, device="cuda:0", generator=gen).to(torch.bfloat16),
+                         ddt=torch.randn(b, l, h, device="cuda:0", generator=gen).to(torch.bfloat16)))
+    w = torch.ones(d, device="cuda:0")
+    bias = torch.zeros(h, device="cuda:0")
+    dpacked = torch.empty(b, l, width, dtype=torch.bfloat16, device="cuda:0")
+    state = {"i": 0}
+
+    def step():
+        s_ = sets[state["i"] % nsets]
+        state["i"] += 1
+        z, dt = s_["packed"][..., :d], s_["packed"][..., width - h:]
+        glue.softplus_bias_hip(dt, bias)
+        glue.rmsnorm_gated_hip(s_["x"], z, w, g, 1e-5, out_dtype=torch.bfloat16)
+        glue.rmsnorm_gated_bwd_hip(s_["x"], z, w, s_["dout"], g, 1e-5, out_dz=dpacked[..., :d])
+        glue.softplus_bias_bwd_hip(dt, bias, s_["ddt"], out_d_in=dpacked[..., width - h:])
+
+    wall_ms, per = event_time_ms(step, steps, warmup)
+    ms = sum(per) / len(per)
+    bytes_ = b * l * d * 2 * 8 + b * l * h * 2 * 5      # norm: x, z, out | x, z, d_out, dx, dz; softplus: dt, out | dt, d_out, d_in
+    tokens = b * l
+    return dict(metric="mixer glue (gated RMSNorm + softplus) fwd+bwd tokens/s", value=tokens / (ms * 1e-3), unit="tokens/s", ms_per_step=ms,
+                dtype="bf16 I/O, f32 arithmetic",
+                config={"workload": "gated RMSNorm d5120 g1 + softplus(dt + bias) h80, fwd+bwd, b4 l2048, packed-buffer column slices"},
+                roofline={"bound": "hbm", "achieved": bytes_ / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": GLUE_TRAFFIC_BYTES,
+                          "algorithmic_bytes_per_step": bytes_,
+                          "kernels": "rmsnorm_gated_kernel fwd + bwd, column_sum_kernel, softplus_fwd_kernel, softplus_bwd_kernel"})
 
 
 def bench_decode(steps, warmup):
@@ -190,7 +233,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", choices=["all", "ssd", "conv", "decode", "copy"])
+    ap.add_argument("--workload", default="all", choices=["all", "ssd", "conv", "glue", "decode", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -221,12 +264,14 @@ def main():
         })
     if a.workload in ("all", "conv"):
         other["conv1d"] = bench_conv(a.steps, a.warmup)
+    if a.workload in ("all", "glue"):
+        other["mixer_glue"] = bench_glue(a.steps, a.warmup)
     if a.workload in ("all", "decode"):
         other["decode"] = bench_decode(max(3, a.steps // 4), max(1, a.warmup // 2))
     if a.workload in ("all", "copy"):
         other["stream_copy"] = bench_copy(a.steps, a.warmup)
     if a.workload not in ("all", "ssd"):
-        key = {"conv": "conv1d", "decode": "decode", "copy": "stream_copy"}[a.workload]
+        key = {"conv": "conv1d", "glue": "mixer_glue", "decode": "decode", "copy": "stream_copy"}[a.workload]
         out.update(other.pop(key))
         out.update({"n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "scaling": "weak", "vs_baseline": None, "data": "synthetic"})
         out.setdefault("higher_is_better", True)

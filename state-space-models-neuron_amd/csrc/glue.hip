@@ -31,40 +31,60 @@ softplus_fwd_kernel(const T* __restrict__ dt, int64_t dt_sr, const float* __rest
     out[row * out_sr + h] = from_f32<T>(v < kSoftplusThreshold ? log1pf(__expf(v)) : v);
 }
 
-constexpr int kSpRows = 64;      // rows per workgroup of the softplus backward
-// one thread per head; a workgroup walks kSpRows rows and leaves one partial row of d_bias
+constexpr int kSpRows = 16;      // rows per workgroup of the softplus backward
+// 256 threads = 4 row phases x 64 heads; a workgroup walks kSpRows rows and leaves one partial row of d_bias
 template <typename T>
-__global__ void __launch_bounds__(128)
+__global__ void __launch_bounds__(256)
 softplus_bwd_kernel(const T* __restrict__ dt, int64_t dt_sr, const float* __restrict__ bias, const T* __restrict__ d_out, int64_t do_sr,
                     T* __restrict__ d_in, int64_t di_sr, float* __restrict__ partial, int64_t rows, int64_t nheads) {
+    __shared__ float red[4][64];
+    const int hl = threadIdx.x & 63, ph = threadIdx.x >> 6;
     const int64_t r0 = (int64_t)blockIdx.x * kSpRows;
     const int64_t r1 = r0 + kSpRows < rows ? r0 + kSpRows : rows;
-    for (int64_t h = threadIdx.x; h < nheads; h += 128) {
-        const float bh = bias[h];
+    for (int64_t h0 = 0; h0 < nheads; h0 += 64) {
+        const int64_t h = h0 + hl;
         float acc = 0.f;
-        for (int64_t r = r0; r < r1; ++r) {
-            const float v = to_f32(dt[r * dt_sr + h]) + bh;
-            const float g = to_f32(d_out[r * do_sr + h]) * (v < kSoftplusThreshold ? sigmoid_f(v) : 1.f);
-            const T gt = from_f32<T>(g);
-            d_in[r * di_sr + h] = gt;
-            acc += g;
+        if (h < nheads) {
+            const float bh = bias[h];
+#pragma unroll 4
+            for (int64_t r = r0 + ph; r < r1; r += 4) {
+                const float v = to_f32(dt[r * dt_sr + h]) + bh;
+                const float g = to_f32(d_out[r * do_sr + h]) * (v < kSoftplusThreshold ? sigmoid_f(v) : 1.f);
+                d_in[r * di_sr + h] = from_f32<T>(g);
+                acc += g;
+            }
         }
-        partial[(int64_t)blockIdx.x * nheads + h] = acc;
+        red[ph][hl] = acc;
+        __syncthreads();
+        if (ph == 0 && h < nheads) partial[(int64_t)blockIdx.x * nheads + h] = (red[0][hl] + red[1][hl]) + (red[2][hl] + red[3][hl]);
+        __syncthreads();
     }
 }
 
-// out[c] = sum over the partial rows of partial[row][c], rows in order.  Four row phases per channel, 64 channels per workgroup.
-__global__ void __launch_bounds__(256)
+// out[c] = sum over the partial rows of partial[row][c] in a fixed order: 16 row phases per channel (1024 threads), 64
+// channels per workgroup, the phases added pairwise.
+__global__ void __launch_bounds__(1024)
 column_sum_kernel(const float* __restrict__ partial, float* __restrict__ out, int64_t nrows, int64_t ncols) {
-    __shared__ float red[4][64];
+    __shared__ float red[16][64];
     const int c = threadIdx.x & 63, ph = threadIdx.x >> 6;
     const int64_t col = (int64_t)blockIdx.x * 64 + c;
     float s = 0.f;
-    if (col < ncols)
-        for (int64_t r = ph; r < nrows; r += 4) s += partial[r * ncols + col];
+    if (col < ncols) {
+#pragma unroll 4
+        for (int64_t r = ph; r < nrows; r += 16) s += partial[r * ncols + col];
+    }
     red[ph][c] = s;
     __syncthreads();
-    if (ph == 0 && col < ncols) out[col] = (red[0][c] + red[1][c]) + (red[2][c] + red[3][c]);
+    if (ph == 0 && col < ncols) {
+        float t[16];
+#pragma unroll
+        for (int q = 0; q < 16; ++q) t[q] = red[q][c];
+#pragma unroll
+        for (int w = 8; w >= 1; w >>= 1)
+#pragma unroll
+            for (int q = 0; q < w; ++q) t[q] += t[q + w];
+        out[col] = t[0];
+    }
 }
 
 // ------------------------------------------------------------------------------------------ gated RMSNorm
@@ -86,8 +106,7 @@ template <> struct GlueVec<bf16_t> { static constexpr int V = 8; };
 template <> struct GlueVec<float> { static constexpr int V = 4; };
 
 template <typename T>
-__device__ __forceinline__ void load_vec(const T* p, float (&v)[GlueVec<T>::V]) {
-    const uint4 raw = *reinterpret_cast<const uint4*>(p);
+__device__ __forceinline__ void unpack_vec(const uint4 raw, float (&v)[GlueVec<T>::V]) {
     if constexpr (sizeof(T) == 2) {
         const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
@@ -154,23 +173,40 @@ rmsnorm_gated_kernel(const NormArgs a) {
     const int64_t r1 = r0 + a.rows_per_block < a.rows ? r0 + a.rows_per_block : a.rows;
     int slot = 0;
     // WPG == 4: every wave takes every row of the block (uniform trip count, barriers inside); WPG == 1: wave w takes rows w, w + 4, ...
-    for (int64_t r = r0 + (WPG == 4 ? 0 : wave); r < r1; r += (WPG == 4 ? 1 : 4)) {
-        const T* xr = static_cast<const T*>(a.x) + r * a.x_sr + c0;
-        const T* zr = a.z ? static_cast<const T*>(a.z) + r * a.z_sr + c0 : nullptr;
+    // the raw vectors of the next row are loaded before this row is reduced (the row after the last: the last once more)
+    constexpr int RSTEP = WPG == 4 ? 1 : 4;
+    const bool gated = a.z != nullptr;
+    uint4 rx[NV], rz[NV], rg[BWD ? NV : 1];
+    auto load_row = [&](int64_t r) {
+        const int64_t rr = r < r1 ? r : r1 - 1;
+        const T* xr = static_cast<const T*>(a.x) + rr * a.x_sr + c0;
+        const T* zr = gated ? static_cast<const T*>(a.z) + rr * a.z_sr + c0 : xr;
+        const T* gr = BWD ? static_cast<const T*>(a.g) + rr * a.g_sr + c0 : xr;
+#pragma unroll
+        for (int it = 0; it < NV; ++it) {
+            const int vi = it * TPG + tl;
+            const int64_t off = (int64_t)(vi < nvec ? vi : 0) * V;      // idle lanes read the first vector and ignore it
+            rx[it] = *reinterpret_cast<const uint4*>(xr + off);
+            rz[it] = *reinterpret_cast<const uint4*>(zr + off);
+            if (BWD) rg[it] = *reinterpret_cast<const uint4*>(gr + off);
+        }
+    };
+    const int64_t rfirst = r0 + (WPG == 4 ? 0 : wave);
+    if (rfirst < r1) load_row(rfirst);
+    for (int64_t r = rfirst; r < r1; r += RSTEP) {
+        const bool zr = gated;
         float h[NV][V], xs[BWD ? NV : 1][V], zs[BWD ? NV : 1][V], gs[BWD ? NV : 1][V];
         float ss = 0.f, dot = 0.f;
 #pragma unroll
         for (int it = 0; it < NV; ++it) {
             const int vi = it * TPG + tl;
             float xv[V], zv[V], gv[V];
-            if (vi < nvec) {
-                load_vec<T>(xr + (int64_t)vi * V, xv);
-                if (zr) load_vec<T>(zr + (int64_t)vi * V, zv);
-                if (BWD) load_vec<T>(static_cast<const T*>(a.g) + r * a.g_sr + c0 + (int64_t)vi * V, gv);
-            }
+            unpack_vec<T>(rx[it], xv);
+            unpack_vec<T>(rz[it], zv);
+            if (BWD) unpack_vec<T>(rg[it], gv);
 #pragma unroll
             for (int e = 0; e < V; ++e) {
-                if (vi >= nvec) { xv[e] = 0.f; zv[e] = 0.f; gv[e] = 0.f; }
+                if (vi >= nvec) { xv[e] = 0.f; zv[e] = 0.f; if (BWD) gv[e] = 0.f; }
                 const float gate = zr ? silu_f(zv[e]) : 1.f;
                 h[it][e] = xv[e] * gate;
                 ss += h[it][e] * h[it][e];
@@ -180,6 +216,7 @@ rmsnorm_gated_kernel(const NormArgs a) {
                 }
             }
         }
+        load_row(r + RSTEP);
         group_sum2<WPG>(ss, dot, red, slot);
         slot ^= 1;
         const float var = ss * inv_n + a.eps;
@@ -237,9 +274,10 @@ rmsnorm_gated_kernel(const NormArgs a) {
     }
 }
 
-// rows per workgroup: about 512 workgroups in all, at least 4 rows each
-int64_t norm_rows_per_block(int64_t rows, int64_t groups) {
-    int64_t rb = rows * groups / 512;
+// rows per workgroup: about 512 workgroups in all for the backward (each leaves a partial row of dw), about 2048 for
+// the forward, at least 4 rows each
+int64_t norm_rows_per_block(int64_t rows, int64_t groups, bool bwd) {
+    int64_t rb = rows * groups / (bwd ? 512 : 1024);
     if (rb < 4) rb = 4;
     return (rb + 3) / 4 * 4;
 }
@@ -309,14 +347,14 @@ extern "C" int m2_softplus_bias_bwd(const void* dt, int64_t dt_stride_row, const
         M2_REQUIRE(workspace && workspace_bytes >= m2_softplus_bias_bwd_workspace_bytes(rows, nheads), M2_ERR_WORKSPACE,
                    "softplus_bias_bwd: workspace %zu bytes < %zu needed", workspace_bytes, m2_softplus_bias_bwd_workspace_bytes(rows, nheads));
         float* partial = static_cast<float*>(workspace);
-        M2_DISPATCH_DTYPE(dtype, T, (softplus_bwd_kernel<T><<<(unsigned)nblk, 128, 0, st>>>(
+        M2_DISPATCH_DTYPE(dtype, T, (softplus_bwd_kernel<T><<<(unsigned)nblk, 256, 0, st>>>(
                                          static_cast<const T*>(dt), dt_stride_row, dt_bias, static_cast<const T*>(d_out), d_out_stride_row,
                                          static_cast<T*>(d_in), d_in_stride_row, partial, rows, nheads)));
         int rc = check_launch("softplus_bwd_kernel");
         if (rc) return rc;
     }
     // with no rows the sum is empty: column_sum_kernel writes zeros
-    column_sum_kernel<<<(unsigned)ceil_div(nheads, (int64_t)64), 256, 0, st>>>(static_cast<const float*>(workspace), d_bias, nblk, nheads);
+    column_sum_kernel<<<(unsigned)ceil_div(nheads, (int64_t)64), 1024, 0, st>>>(static_cast<const float*>(workspace), d_bias, nblk, nheads);
     return check_launch("column_sum_kernel");
 }
 
@@ -334,7 +372,7 @@ extern "C" int m2_rmsnorm_gated_fwd(const m2_rmsnorm_params* p, void* stream) {
     a.x = p->x; a.x_sr = p->x_stride_row; a.z = p->z; a.z_sr = p->z_stride_row; a.w = p->weight;
     a.out = p->out; a.out_sr = p->out_stride_row; a.out_f32 = p->out_f32 || p->dtype == M2_F32;
     a.rows = p->rows; a.d = p->channels; a.gw = p->channels / p->n_groups; a.eps = p->eps;
-    a.rows_per_block = norm_rows_per_block(p->rows, p->n_groups);
+    a.rows_per_block = norm_rows_per_block(p->rows, p->n_groups, false);
     hipStream_t st = static_cast<hipStream_t>(stream);
     M2_DISPATCH_DTYPE(p->dtype, T, return (launch_norm<T, false>(a, p->n_groups, st)));
     return M2_OK;
@@ -342,7 +380,7 @@ extern "C" int m2_rmsnorm_gated_fwd(const m2_rmsnorm_params* p, void* stream) {
 
 extern "C" size_t m2_rmsnorm_gated_bwd_workspace_bytes(int64_t rows, int64_t channels, int32_t n_groups, int32_t dtype) {
     if (rows <= 0 || channels <= 0 || n_groups <= 0) return 256;
-    const int64_t nrb = m2::ceil_div(rows, m2::norm_rows_per_block(rows, n_groups));
+    const int64_t nrb = m2::ceil_div(rows, m2::norm_rows_per_block(rows, n_groups, true));
     return m2::align_up((size_t)nrb * 4 * (size_t)channels * sizeof(float), 256);      // up to one partial row per wave
 }
 
@@ -370,7 +408,7 @@ extern "C" int m2_rmsnorm_gated_bwd(const m2_rmsnorm_params* p, void* stream) {
         a.g = p->d_out; a.g_sr = p->d_out_stride_row; a.dx = p->dx; a.dx_sr = p->dx_stride_row; a.dz = p->dz; a.dz_sr = p->dz_stride_row;
         a.partial = static_cast<float*>(p->workspace);
         a.rows = p->rows; a.d = p->channels; a.gw = p->channels / p->n_groups; a.eps = p->eps;
-        a.rows_per_block = norm_rows_per_block(p->rows, p->n_groups);
+        a.rows_per_block = norm_rows_per_block(p->rows, p->n_groups, true);
         int wpg = 0, nv = 0;
         if (!norm_shape(a.gw / V, &wpg, &nv))
             return fail(M2_ERR_SHAPE, "rmsnorm_gated_bwd: %lld channels per group exceed the supported %d", (long long)a.gw, 1024 * V);
@@ -378,7 +416,7 @@ extern "C" int m2_rmsnorm_gated_bwd(const m2_rmsnorm_params* p, void* stream) {
         M2_DISPATCH_DTYPE(p->dtype, T, rc = (launch_norm<T, true>(a, p->n_groups, st)));
         if (rc) return rc;
     }
-    column_sum_kernel<<<(unsigned)ceil_div(p->channels, (int64_t)64), 256, 0, st>>>(static_cast<const float*>(p->workspace), p->d_weight,
+    column_sum_kernel<<<(unsigned)ceil_div(p->channels, (int64_t)64), 1024, 0, st>>>(static_cast<const float*>(p->workspace), p->d_weight,
                                                                                      prows, p->channels);
     return check_launch("column_sum_kernel");
 }
