@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0              # MI355X HBM3E
 SSD_TRAFFIC_BYTES = 1.441e9
 CONV_TRAFFIC_BYTES = 459.5e6
 DECODE_TRAFFIC_BYTES = 64 * 689.3e6
-GLUE_TRAFFIC_BYTES = None
+GLUE_TRAFFIC_BYTES = 703.5e6
 
 SSD_CFG = dict(b=4, l=2048, h=80, p=64, n=128, g=1)
 CONV_CFG = dict(b=4, l=2048, C=5376, k=4)

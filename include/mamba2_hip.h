@@ -13,7 +13,7 @@
  *                                         :277-485 (mamba_kernel_bwd_); wrapper :488-519
  *   m2_decode_step                     <- mamba2/mamba2_kernel_inference.py:27-104
  *                                         (mamba_inference_kernel_); wrapper :107-122
- *   m2_softplus_bias_* / m2_rmsnorm_gated_*  <- mamba2/fused_kernel.py:24-175 (glue kernels of the
+ *   m2_softplus_bias_* / m2_rmsnorm_gated_*  <- mamba2/fused_kernel.py:33-175 (glue kernels of the
  *                                         fused mixer core)
  *
  * Conventions
@@ -154,8 +154,8 @@ int m2_decode_step(const m2_decode_params* p, void* stream);
 
 /* ------------------------------------------------------------------ mixer glue
  * The elementwise passes between the conv, the scan and the output projection
- * (mamba2/fused_kernel.py:24-47 softplus_with_bias, :50-73 softplus_with_bias_bwd,
- * :76-105 rmsnorm, :128-175 rmsnorm_bwd; torch twins mamba2/mamba2_mixer.py:36-38, 88-105).
+ * (mamba2/fused_kernel.py:33-47 softplus_with_bias, :50-73 softplus_with_bias_bwd,
+ * :76-103 rmsnorm, :127-175 rmsnorm_bwd; torch twins mamba2/mamba2_mixer.py:36-38, 88-105).
  * Rows are (batch x token) pairs; the channel dimension is contiguous, rows may be strided
  * (columns of the packed [z | xBC | dt] projection output and of its gradient).
  *

@@ -1,5 +1,5 @@
 // Elementwise glue of the mixer core as HBM-bound kernels: softplus(dt + dt_bias) and the gated, grouped RMSNorm,
-// forward and backward (mamba2/fused_kernel.py:24-73 softplus_with_bias(_bwd), :76-175 rmsnorm(_bwd); torch twins
+// forward and backward (mamba2/fused_kernel.py:33-73 softplus_with_bias(_bwd), :76-175 rmsnorm(_bwd); torch twins
 // mamba2/mamba2_mixer.py:36-38, 88-105).  Every tensor is read once and written once; all arithmetic is fp32.
 //
 //   softplus:  out = v < 10 ? log(1 + e^v) : v,  v = dt + bias[h]              (threshold form, mamba2_mixer.py:36-38)
