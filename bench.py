@@ -153,6 +153,42 @@ def bench_glue(steps, warmup):
                           "kernels": "rmsnorm_gated_kernel fwd + bwd, column_sum_kernel, softplus_fwd_kernel, softplus_bwd_kernel"})
 
 
+def bench_core(steps, warmup):
+    """The fused mixer core zxBCdt -> norm_out (conv + SiLU, softplus, SSD scan, gated norm) forward + backward at the
+    2.7B layer shape, through the reference's autograd-function signature (the caching variant: nothing is recomputed)."""
+    import torch
+    from mamba2.fused_kernel import mamba2_fused_kernel_with_caching
+    cfg = SSD_CFG
+    b, l, h, p, n, g = cfg["b"], cfg["l"], cfg["h"], cfg["p"], cfg["n"], cfg["g"]
+    d = h * p
+    width = 2 * d + 2 * g * n + h
+    gen = torch.Generator(device="cuda:0").manual_seed(0)
+    zx = torch.randn(b, l, width, device="cuda:0", generator=gen)
+    zx[..., 2 * d:2 * d + 2 * g * n] /= n ** 0.5
+    zx = zx.to(torch.bfloat16).requires_grad_(True)
+    A = (-torch.exp(torch.empty(h, device="cuda:0").uniform_(0.0, 2.77, generator=gen))).requires_grad_(True)
+    D = torch.ones(h, device="cuda:0", requires_grad=True)
+    cw = (torch.rand(d + 2 * g * n, 1, 4, device="cuda:0", generator=gen) - 0.5).to(torch.bfloat16).requires_grad_(True)
+    cb = (torch.rand(d + 2 * g * n, device="cuda:0", generator=gen) - 0.5).to(torch.bfloat16).requires_grad_(True)
+    dtb = torch.empty(h, device="cuda:0").uniform_(-5.0, -2.0, generator=gen).requires_grad_(True)
+    nw = torch.ones(d, device="cuda:0", requires_grad=True)
+    dout = torch.randn(b, l, d, device="cuda:0", generator=gen).to(torch.bfloat16)
+    leaves = (zx, A, D, cw, cb, dtb, nw)
+
+    def step():
+        for t in leaves:
+            t.grad = None
+        out = mamba2_fused_kernel_with_caching(zx, A, D, cw, cb, dtb, nw, g, n, d, p)
+        out.backward(dout)
+
+    wall_ms, per = event_time_ms(step, steps, warmup)
+    ms = sum(per) / len(per)
+    tokens = b * l
+    return dict(metric="fused mixer core fwd+bwd tokens/s", value=tokens / (wall_ms * 1e-3), unit="tokens/s", ms_per_step=wall_ms,
+                event_ms_avg=ms, dtype="bf16",
+                config={"workload": "mamba2_fused_kernel_with_caching fwd+bwd, zxBCdt (4, 2048, 10576): conv k4 + SiLU, softplus, SSD h80 p64 n128 g1, gated RMSNorm"})
+
+
 def bench_decode(steps, warmup):
     import torch
     from mamba2.mamba2_kernel_inference import mamba2_kernel_inference
@@ -233,7 +269,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", choices=["all", "ssd", "conv", "glue", "decode", "copy"])
+    ap.add_argument("--workload", default="all", choices=["all", "ssd", "conv", "glue", "core", "decode", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -266,12 +302,14 @@ def main():
         other["conv1d"] = bench_conv(a.steps, a.warmup)
     if a.workload in ("all", "glue"):
         other["mixer_glue"] = bench_glue(a.steps, a.warmup)
+    if a.workload in ("all", "core"):
+        other["mixer_core"] = bench_core(a.steps, a.warmup)
     if a.workload in ("all", "decode"):
         other["decode"] = bench_decode(max(3, a.steps // 4), max(1, a.warmup // 2))
     if a.workload in ("all", "copy"):
         other["stream_copy"] = bench_copy(a.steps, a.warmup)
     if a.workload not in ("all", "ssd"):
-        key = {"conv": "conv1d", "glue": "mixer_glue", "decode": "decode", "copy": "stream_copy"}[a.workload]
+        key = {"conv": "conv1d", "glue": "mixer_glue", "core": "mixer_core", "decode": "decode", "copy": "stream_copy"}[a.workload]
         out.update(other.pop(key))
         out.update({"n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "scaling": "weak", "vs_baseline": None, "data": "synthetic"})
         out.setdefault("higher_is_better", True)
