@@ -79,8 +79,9 @@ def bench_ssd(steps, warmup):
     ms = sum(per) / len(per)
     tokens = cfg["b"] * cfg["l"]
     flops = 3 * ssd_flops_fwd(**cfg)
+    io_bytes = 2 * (5 * cfg["b"] * cfg["l"] * cfg["h"] * cfg["p"] + 4 * cfg["b"] * cfg["l"] * cfg["g"] * cfg["n"] + 2 * cfg["b"] * cfg["l"] * cfg["h"])
     return dict(ms_per_step=wall_ms, ms_event_avg=ms, ms_event_min=per[0], ms_event_median=per[len(per) // 2],
-                tokens_per_s=tokens / (wall_ms * 1e-3), flops=flops, tflops=flops / (ms * 1e-3) / 1e12, tokens=tokens)
+                tokens_per_s=tokens / (wall_ms * 1e-3), flops=flops, io_bytes=io_bytes, tflops=flops / (ms * 1e-3) / 1e12, tokens=tokens)
 
 
 def bench_conv(steps, warmup):
@@ -297,6 +298,10 @@ def main():
                          "algorithmic_flops_per_step": r["flops"], "event_ms_avg": r["ms_event_avg"],
                          "event_ms_min": r["ms_event_min"],
                          "kernels": "all launches of m2_ssd_fwd + m2_ssd_bwd (one step), HIP events on the launch stream"},
+            # the same step against the memory roofline: algorithmic I/O = x (forward), y, x (backward), dy, dx, B, C, dB, dC, dt, ddt
+            "roofline_hbm": {"bound": "hbm", "achieved": r["io_bytes"] / (r["ms_event_avg"] * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": r["io_bytes"] / (r["ms_event_avg"] * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": SSD_TRAFFIC_BYTES,
+                             "traffic_rate": SSD_TRAFFIC_BYTES / (r["ms_event_avg"] * 1e-3) / 1e9, "algorithmic_bytes_per_step": r["io_bytes"]},
         })
     if a.workload in ("all", "conv"):
         other["conv1d"] = bench_conv(a.steps, a.warmup)

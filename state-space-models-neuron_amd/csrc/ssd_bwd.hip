@@ -28,11 +28,12 @@
 // Launch sequence (16-bit operands; fp32 operands take the kernels named in brackets):
 //   prep_kernel, state_pass16_kernel [chunk_state + state_scan]   recompute G, tables, S_prev (skipped if the caller kept them)
 //   state_pass16_kernel<REVERSE> [chunk_state<DSTATE> + state_scan<REVERSE>]
-//                                                              dS per chunk, e^{Lam} <dS, S_prev>, d initial state
+//                                                              dS per chunk, d initial state (and e^{Lam} <dS, S_prev> when
+//                                                              ssd_bwd16_kernel does not run)
 //   dg16_kernel [dg_kernel]   per (b, chunk, group, head slice)  partial dG (heads reduced in registers), dl_diag per head
 //   ssd_bwd16_kernel [off_kernel<C>, <B>, diag_off_kernel<bwd>]
-//                             per (b, chunk, group, head slice)  dx, per-token decay-gradient terms, dD partials,
-//                                                                partial state parts of dB / dC
+//                             per (b, chunk, group, head slice)  dx, per-token decay-gradient terms, e^{Lam} <dS, S_prev>,
+//                                                                dD partials, partial state parts of dB / dC
 //   tail1_kernel              da_body: ddt, dA partials per (b, head, chunk);  slice_sum_body: partials over the head slices
 //   tail2_kernel              bc_final_body per (b, chunk, group): dC = dG B + dCoff, dB = dG^T C + dBoff;
 //                             ad_reduce_body per head: dA, dD (fixed order, no atomics)
