@@ -100,6 +100,11 @@ int m2_conv1d_bwd(const m2_conv1d_params* p, void* stream);
  * into the workspace).  Backward: if non-NULL it must hold what the forward wrote for the same
  * inputs and is read instead of being recomputed; with NULL the backward recomputes all of it
  * from the inputs, as the reference does (mamba2_kernel.py:363-367).
+ * dt_bias (optional, (h) fp32): when given, `dt` holds the RAW projection output and the step
+ * size is softplus(dt + dt_bias[h]) (threshold form, x for x >= 10), applied where the decay
+ * tables are built -- the fused mixer core's softplus_with_bias (fused_kernel.py:33-47, called at
+ * :273) without a pass of its own.  The backward then returns ddt w.r.t. the raw dt and
+ * d_dt_bias (h) fp32 summed over batch and tokens (softplus_with_bias_bwd, :50-73).
  */
 typedef struct m2_ssd_params {
     const void* x; const void* dt; const float* A; const void* B; const void* C; const float* D;
@@ -123,6 +128,8 @@ typedef struct m2_ssd_params {
     int64_t dC_stride_b, dC_stride_l, dC_stride_g;
     int32_t dtype;                                      /* x, B, C, y, dy, dx, dB, dC   */
     int32_t dt_dtype;                                   /* dt, ddt                      */
+    const float* dt_bias;                               /* optional (h): see below      */
+    float* d_dt_bias;                                   /* backward, with dt_bias: (h)  */
 } m2_ssd_params;
 
 size_t m2_ssd_chunk_states_bytes(const m2_ssd_params* p);

@@ -105,6 +105,12 @@ __device__ __forceinline__ float silu_grad_f(float z) {
     return s * (1.0f + z * (1.0f - s));
 }
 
+// softplus in the threshold form of the reference's torch twin (mamba2/mamba2_mixer.py:36-38): x itself from 10 on.
+constexpr float kSoftplusThreshold = 10.0f;
+__device__ __forceinline__ float softplus_f(float v) { return v < kSoftplusThreshold ? log1pf(__expf(v)) : v; }
+// d softplus / dv expressed through the VALUE s = softplus(v): sigmoid(v) = 1 - e^{-s} (1 from the threshold on)
+__device__ __forceinline__ float softplus_grad_of_value(float s) { return s < kSoftplusThreshold ? -expm1f(-s) : 1.f; }
+
 template <int ACT> __device__ __forceinline__ float act_f(float z) {
     if (ACT == M2_ACT_SILU) return silu_f(z);
     if (ACT == M2_ACT_RELU) return z > 0.f ? z : 0.f;

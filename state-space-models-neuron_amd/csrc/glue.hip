@@ -17,8 +17,6 @@
 namespace m2 {
 namespace {
 
-constexpr float kSoftplusThreshold = 10.0f;
-
 // ------------------------------------------------------------------------------------------ softplus
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -28,7 +26,7 @@ softplus_fwd_kernel(const T* __restrict__ dt, int64_t dt_sr, const float* __rest
     if (idx >= rows * nheads) return;
     const int64_t row = idx / nheads, h = idx % nheads;
     const float v = to_f32(dt[row * dt_sr + h]) + bias[h];
-    out[row * out_sr + h] = from_f32<T>(v < kSoftplusThreshold ? log1pf(__expf(v)) : v);
+    out[row * out_sr + h] = from_f32<T>(softplus_f(v));
 }
 
 constexpr int kSpRows = 16;      // rows per workgroup of the softplus backward

@@ -432,25 +432,28 @@ bc_final_body(const float* __restrict__ dGp, const float* __restrict__ dCp, cons
 }
 
 // dA[h] = sum_{b,c} dAp[b][h][c], dD likewise (fixed order, no atomics).  One workgroup of 512 threads per head.
-__device__ __forceinline__ void ad_reduce_body(const float* __restrict__ dAp, const float* __restrict__ dDp, float* __restrict__ dA,
-                                               float* __restrict__ dD, int64_t nb, int64_t nheads, int64_t nchunks, int64_t h) {
-    __shared__ float red[2][8];
-    float sa = 0.f, sd = 0.f;
+__device__ __forceinline__ void ad_reduce_body(const float* __restrict__ dAp, const float* __restrict__ dDp, const float* __restrict__ dbp,
+                                               float* __restrict__ dA, float* __restrict__ dD, float* __restrict__ dbias,
+                                               int64_t nb, int64_t nheads, int64_t nchunks, int64_t h) {
+    __shared__ float red[3][8];
+    float sa = 0.f, sd = 0.f, sb = 0.f;
     for (int64_t e = threadIdx.x; e < nb * nchunks; e += 512) {
         const int64_t b = e / nchunks, c = e % nchunks;
         sa += dAp[(b * nheads + h) * nchunks + c];
         sd += dDp[(b * nheads + h) * nchunks + c];
+        if (dbias) sb += dbp[(b * nheads + h) * nchunks + c];
     }
-    sa = warp_sum(sa); sd = warp_sum(sd);
+    sa = warp_sum(sa); sd = warp_sum(sd); sb = warp_sum(sb);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    if (lane == 0) { red[0][wave] = sa; red[1][wave] = sd; }
+    if (lane == 0) { red[0][wave] = sa; red[1][wave] = sd; red[2][wave] = sb; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        float ta = 0.f, td = 0.f;
+        float ta = 0.f, td = 0.f, tb = 0.f;
 #pragma unroll
-        for (int q = 0; q < 8; ++q) { ta += red[0][q]; td += red[1][q]; }
+        for (int q = 0; q < 8; ++q) { ta += red[0][q]; td += red[1][q]; tb += red[2][q]; }
         dA[h] = ta;
         if (dD) dD[h] = td;
+        if (dbias) dbias[h] = tb;
     }
 }
 
@@ -460,7 +463,7 @@ __device__ __forceinline__ void ad_reduce_body(const float* __restrict__ dAp, co
 struct Tail2Args {
     const float* dGp; const float* dCp; const float* dBp; const void* Bt; const void* Ct; void* dB; void* dC;
     int64_t dBsb, dBsl, dBsg, dCsb, dCsl, dCsg;
-    const float* dAp; const float* dDp; float* dA; float* dD;
+    const float* dAp; const float* dDp; const float* dbp; float* dA; float* dD; float* dbias;
     int64_t seqlen, ngroups, nchunks, batch, nheads, n_bc;
 };
 template <typename T, int N>
@@ -474,7 +477,7 @@ tail2_kernel(const Tail2Args a) {
                             static_cast<T*>(a.dC), a.seqlen, a.ngroups, a.nchunks, a.dBsb, a.dBsl, a.dBsg, a.dCsb, a.dCsl, a.dCsg, c, g, b,
                             (blk & 1) != 0);
     } else {
-        ad_reduce_body(a.dAp, a.dDp, a.dA, a.dD, a.batch, a.nheads, a.nchunks, blk - 2 * a.n_bc);
+        ad_reduce_body(a.dAp, a.dDp, a.dbp, a.dA, a.dD, a.dbias, a.batch, a.nheads, a.nchunks, blk - 2 * a.n_bc);
     }
 }
 
@@ -591,6 +594,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         a.ddt = p->ddt; a.ddt_sb = p->ddt_stride_b; a.ddt_sl = p->ddt_stride_l;
         a.ldtab = w.ldtab;
         a.dl_diag = w.dl; a.dl_c = w.dlc; a.dlam = w.dlam; a.dAp = w.dAp; a.dDp = w.dDp;
+        a.dbp = p->dt_bias ? w.dbp : nullptr;
         const dim3 grid((unsigned)nc, (unsigned)(p->ngroups * a.nslices), (unsigned)p->batch);
         if constexpr (bwd16_ok<T, P, N>()) {
             Bwd16Args m{};
@@ -614,6 +618,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
             da.ldtab = w.ldtab; da.A = p->A; da.dl_diag = w.dl; da.dl_c = w.dlc; da.dlam = w.dlam;
             da.dirp = w.dirp; da.rbp = w.rbp; da.dDp8 = w.dDp8;
             da.ddt = p->ddt; da.dt_f32 = dt_f32; da.ddt_sb = p->ddt_stride_b; da.ddt_sl = p->ddt_stride_l; da.dAp = w.dAp; da.dDp = w.dDp;
+            da.dbp = p->dt_bias ? w.dbp : nullptr;
             da.seqlen = p->seqlen; da.nheads = p->nheads; da.nchunks = nc; da.total = p->batch * p->nheads * nc;
         } else {
             auto k = diag_off_kernel<T, P, N, true>;
@@ -651,7 +656,8 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         ta.dGp = gs; ta.dCp = cs; ta.dBp = bs; ta.Bt = w.Bt; ta.Ct = w.Ct; ta.dB = p->dB; ta.dC = p->dC;
         ta.dBsb = p->dB_stride_b; ta.dBsl = p->dB_stride_l; ta.dBsg = p->dB_stride_g;
         ta.dCsb = p->dC_stride_b; ta.dCsl = p->dC_stride_l; ta.dCsg = p->dC_stride_g;
-        ta.dAp = w.dAp; ta.dDp = w.dDp; ta.dA = p->dA; ta.dD = p->D ? p->dD : nullptr;
+        ta.dAp = w.dAp; ta.dDp = w.dDp; ta.dbp = w.dbp; ta.dA = p->dA; ta.dD = p->D ? p->dD : nullptr;
+        ta.dbias = p->dt_bias ? p->d_dt_bias : nullptr;
         ta.seqlen = p->seqlen; ta.ngroups = p->ngroups; ta.nchunks = nc; ta.batch = p->batch; ta.nheads = p->nheads; ta.n_bc = ngrp;
         k<<<(unsigned)(2 * ngrp + p->nheads), 512, sm, st>>>(ta);
         if ((rc = check_launch("ssd tail2_kernel"))) return rc;
@@ -675,10 +681,12 @@ extern "C" int m2_ssd_bwd(const m2_ssd_params* p, void* stream) {
     if (p->nheads == 0) return M2_OK;
     M2_REQUIRE(p->dA, M2_ERR_NULL, "ssd_bwd: dA is required");
     M2_REQUIRE(!p->D || p->dD, M2_ERR_NULL, "ssd_bwd: dD is required when D is given");
+    M2_REQUIRE(!p->dt_bias || p->d_dt_bias, M2_ERR_NULL, "ssd_bwd: d_dt_bias is required when dt_bias is given");
     if (p->batch == 0 || p->seqlen == 0) {
         // empty reductions: parameter gradients are zero; the state gradient passes straight through
         zero_f32_kernel<<<(unsigned)ceil_div(p->nheads, (int64_t)256), 256, 0, st>>>(p->dA, p->nheads);
         if (p->dD) zero_f32_kernel<<<(unsigned)ceil_div(p->nheads, (int64_t)256), 256, 0, st>>>(p->dD, p->nheads);
+        if (p->dt_bias) zero_f32_kernel<<<(unsigned)ceil_div(p->nheads, (int64_t)256), 256, 0, st>>>(p->d_dt_bias, p->nheads);
         if (p->d_initial_state && p->batch > 0) {
             const int64_t n = p->batch * p->nheads * p->headdim * p->dstate;
             copy_f32_kernel<<<(unsigned)ceil_div(n, (int64_t)256), 256, 0, st>>>(p->d_final_state, p->d_initial_state, n);

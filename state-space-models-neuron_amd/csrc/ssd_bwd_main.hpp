@@ -414,6 +414,7 @@ struct DaArgs {
     const float* ldtab; const float* A; const float* dl_diag; const float* dl_c; const float* dlam;
     const float* dirp; const float* rbp; const float* dDp8;
     void* ddt; int dt_f32; int64_t ddt_sb, ddt_sl; float* dAp; float* dDp;
+    float* dbp;            // with softplus folded into the scan: [b][h][c] partials of d_dt_bias, and ddt is w.r.t. the raw dt; else null
     int64_t seqlen, nheads, nchunks, total;
 };
 template <typename T>
@@ -422,7 +423,7 @@ __device__ __forceinline__ void da_body(const DaArgs& q, int64_t blk) {
     const float* __restrict__ dl_diag = q.dl_diag; const float* __restrict__ dl_c = q.dl_c; const float* __restrict__ dlam = q.dlam;
     const float* __restrict__ dirp = q.dirp; const float* __restrict__ rbp = q.rbp; const float* __restrict__ dDp8 = q.dDp8;
     void* __restrict__ ddt = q.ddt; const int dt_f32 = q.dt_f32; const int64_t ddt_sb = q.ddt_sb, ddt_sl = q.ddt_sl;
-    float* __restrict__ dAp = q.dAp; float* __restrict__ dDp = q.dDp;
+    float* __restrict__ dAp = q.dAp; float* __restrict__ dDp = q.dDp; float* __restrict__ dbp = q.dbp;
     const int64_t seqlen = q.seqlen, nheads = q.nheads, nchunks = q.nchunks, total = q.total;
     const int lane = threadIdx.x & 63;
     const int64_t bhc = blk * 4 + (threadIdx.x >> 6);
@@ -452,22 +453,26 @@ __device__ __forceinline__ void da_body(const DaArgs& q, int64_t blk) {
     xa += (ya - ra) + __shfl(yb, 0, 64);
     xb += yb - rbv;
     const float da_a = xa + dlm, da_b = xb + dlm;
-    float dAl = 0.f;
+    float dAl = 0.f, dbl = 0.f;
     if (ta < valid) {
-        const float val = Ah * da_a + dira;
+        float val = Ah * da_a + dira;
+        if (dbp) { val *= softplus_grad_of_value(dta); dbl += val; }      // dta = softplus(raw dt + bias)
         const int64_t oo = b * ddt_sb + (t0 + ta) * ddt_sl + h;
         if (dt_f32) static_cast<float*>(ddt)[oo] = val; else static_cast<T*>(ddt)[oo] = from_f32<T>(val);
         dAl += da_a * dta;
     }
     if (tb < valid) {
-        const float val = Ah * da_b + dirb;
+        float val = Ah * da_b + dirb;
+        if (dbp) { val *= softplus_grad_of_value(dtb); dbl += val; }
         const int64_t oo = b * ddt_sb + (t0 + tb) * ddt_sl + h;
         if (dt_f32) static_cast<float*>(ddt)[oo] = val; else static_cast<T*>(ddt)[oo] = from_f32<T>(val);
         dAl += da_b * dtb;
     }
     dAl = warp_sum(dAl);
+    if (dbp) dbl = warp_sum(dbl);
     if (lane == 0) {
         dAp[bhc] = dAl;
+        if (dbp) dbp[bhc] = dbl;
         float s = 0.f;
 #pragma unroll
         for (int w = 0; w < 8; ++w) s += dDp8[bhc * 8 + w];

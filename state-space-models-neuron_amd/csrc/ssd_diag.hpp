@@ -46,6 +46,7 @@ struct DiagArgs {
     void* ddt; int64_t ddt_sb, ddt_sl;
     const float* dl_diag; const float* dl_c; const float* dlam;   // [b][h][c][kQ], [b][h][c][kQ], [b][h][c]
     float* dAp; float* dDp;                                       // [b][h][c]
+    float* dbp;            // softplus folded into the scan: [b][h][c] partials of d_dt_bias (ddt is then w.r.t. the raw dt), else null
 };
 
 // The backward keeps a transposed copy of x in LDS for its epilogue when that fits (always for bf16);
@@ -318,21 +319,25 @@ diag_off_kernel(const DiagArgs a) {
 #pragma unroll
                 for (int sp = 0; sp < kDlamParts; ++sp) dlm += a.dlam[bhc * kDlamParts + sp];
                 const float da_a = xa + dlm, da_b = xb + dlm;
-                float dAl = 0.f;
+                float dAl = 0.f, dbl = 0.f;
                 if (ta < valid) {
-                    const float val = Ah * da_a + s_dir[ta];
+                    float val = Ah * da_a + s_dir[ta];
+                    if (a.dbp) { val *= softplus_grad_of_value(wd[ta]); dbl += val; }      // wd = softplus(raw dt + bias)
                     const int64_t o = b * a.ddt_sb + (t0 + ta) * a.ddt_sl + h;
                     if (a.dt_f32) static_cast<float*>(a.ddt)[o] = val; else static_cast<T*>(a.ddt)[o] = from_f32<T>(val);
                     dAl += da_a * wd[ta];
                 }
                 if (tb < valid) {
-                    const float val = Ah * da_b + s_dir[tb];
+                    float val = Ah * da_b + s_dir[tb];
+                    if (a.dbp) { val *= softplus_grad_of_value(wd[tb]); dbl += val; }
                     const int64_t o = b * a.ddt_sb + (t0 + tb) * a.ddt_sl + h;
                     if (a.dt_f32) static_cast<float*>(a.ddt)[o] = val; else static_cast<T*>(a.ddt)[o] = from_f32<T>(val);
                     dAl += da_b * wd[tb];
                 }
                 dAl = warp_sum(dAl);
+                if (a.dbp) dbl = warp_sum(dbl);
                 if (lane == 0) {
+                    if (a.dbp) a.dbp[bhc] = dbl;
                     a.dAp[bhc] = dAl;
                     a.dDp[bhc] = s_red[0] + s_red[1] + s_red[2] + s_red[3];
                 }

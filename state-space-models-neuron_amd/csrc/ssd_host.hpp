@@ -17,6 +17,7 @@ struct SsdWorkspace {
     void* Gm = nullptr; void* Gmt = nullptr; void* Bt = nullptr; void* Ct = nullptr;
     float* ldtab = nullptr;             // [b][h][c][ l kQ | dt kQ ]
     void* dprev = nullptr; float* dlam = nullptr;
+    float* dbp = nullptr;                                               // per (b, h, chunk) partials of d_dt_bias
     float* dAp = nullptr; float* dDp = nullptr; float* dBp = nullptr; float* dCp = nullptr; float* dl = nullptr; float* dlc = nullptr; float* dGp = nullptr;
     float* dGs = nullptr; float* dBs = nullptr; float* dCs = nullptr;   // partials summed over the head slices
     float* dirp = nullptr; float* rbp = nullptr; float* dDp8 = nullptr; // per channel-half / per-wave partials of the dx kernel
@@ -101,6 +102,7 @@ inline SsdWorkspace ssd_carve(const m2_ssd_params* p, void* base, bool bwd, bool
         w.dlam = reinterpret_cast<float*>(take(bhc * 4 * kDlamParts));
         w.dAp = reinterpret_cast<float*>(take(bhc * 4));
         w.dDp = reinterpret_cast<float*>(take(bhc * 4));
+        w.dbp = reinterpret_cast<float*>(take(bhc * 4));
         w.dl = reinterpret_cast<float*>(take(bhc * kQ * 4));
         w.dlc = reinterpret_cast<float*>(take(bhc * kQ * 4));
         w.dirp = reinterpret_cast<float*>(take(bhc * 2 * kQ * 4));
@@ -173,7 +175,7 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
         pa.Bm = Bm; pa.Cm = Cm; pa.Gf = w.G; pa.Gm = w.Gm; pa.Gmt = w.Gmt; pa.Bt = w.Bt; pa.Ct = w.Ct;
         pa.Bsb = p->B_stride_b; pa.Bsl = p->B_stride_l; pa.Bsg = p->B_stride_g;
         pa.Csb = p->C_stride_b; pa.Csl = p->C_stride_l; pa.Csg = p->C_stride_g;
-        pa.dt = p->dt; pa.dt_f32 = dt_f32; pa.A = p->A; pa.ldtab = w.ldtab; pa.lam = w.lam;
+        pa.dt = p->dt; pa.dt_f32 = dt_f32; pa.dt_bias = p->dt_bias; pa.A = p->A; pa.ldtab = w.ldtab; pa.lam = w.lam;
         pa.dtsb = p->dt_stride_b; pa.dtsl = p->dt_stride_l;
         pa.seqlen = p->seqlen; pa.nheads = p->nheads; pa.ngroups = p->ngroups; pa.nchunks = nc;
         pa.total_bhc = p->batch * p->nheads * nc;

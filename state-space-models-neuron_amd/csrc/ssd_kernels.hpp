@@ -121,7 +121,7 @@ cb_body(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict__ 
 // of gathering dt (stride = nheads elements) and scanning it again per head.
 template <typename T>
 __device__ __forceinline__ void
-ld_table_body(const void* __restrict__ dt, int dt_f32, const float* __restrict__ A, float* __restrict__ ldtab,
+ld_table_body(const void* __restrict__ dt, int dt_f32, const float* __restrict__ dt_bias, const float* __restrict__ A, float* __restrict__ ldtab,
               float* __restrict__ lam, int64_t seqlen, int64_t nheads, int64_t nchunks, int64_t total,
               int64_t dtsb, int64_t dtsl, int64_t blk) {
     const int lane = threadIdx.x & 63;
@@ -131,7 +131,14 @@ ld_table_body(const void* __restrict__ dt, int dt_f32, const float* __restrict__
     const int64_t t0 = c * kQ;
     const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
     float l0, l1, d0, d1;
-    wave_chunk_cumsum<T>(dt, dt_f32, b * dtsb + t0 * dtsl + h, dtsl, valid, A[h], l0, l1, d0, d1);
+    wave_dt_load<T>(dt, dt_f32, b * dtsb + t0 * dtsl + h, dtsl, valid, d0, d1);
+    if (dt_bias) {
+        // dt holds the raw projection: the step size is softplus(dt + dt_bias) (0 stays 0 past the end of the sequence)
+        const float bh = dt_bias[h];
+        if (lane < valid) d0 = softplus_f(d0 + bh);
+        if (lane + 64 < valid) d1 = softplus_f(d1 + bh);
+    }
+    wave_cumsum_from(A[h], d0, d1, l0, l1);
     float* p = ldtab + bhc * (2 * kQ);
     p[lane] = l0; p[lane + 64] = l1; p[kQ + lane] = d0; p[kQ + lane + 64] = d1;
     if (lane == 63) lam[bhc] = l1;
@@ -142,7 +149,7 @@ ld_table_body(const void* __restrict__ dt, int dt_f32, const float* __restrict__
 struct PrepArgs {
     const void* Bm; const void* Cm; float* Gf; void* Gm; void* Gmt; void* Bt; void* Ct;
     int64_t Bsb, Bsl, Bsg, Csb, Csl, Csg;
-    const void* dt; int dt_f32; const float* A; float* ldtab; float* lam; int64_t dtsb, dtsl;
+    const void* dt; int dt_f32; const float* dt_bias; const float* A; float* ldtab; float* lam; int64_t dtsb, dtsl;
     int64_t seqlen, nheads, ngroups, nchunks, total_bhc, n_cb;
 };
 template <typename T, int N>
@@ -156,7 +163,7 @@ prep_kernel(const PrepArgs a) {
                       static_cast<T*>(a.Bt), static_cast<T*>(a.Ct), a.seqlen, a.ngroups, a.nchunks,
                       a.Bsb, a.Bsl, a.Bsg, a.Csb, a.Csl, a.Csg, c, g, b, (int)(blk % kCbParts));
     } else {
-        ld_table_body<T>(a.dt, a.dt_f32, a.A, a.ldtab, a.lam, a.seqlen, a.nheads, a.nchunks, a.total_bhc, a.dtsb, a.dtsl, blk - kCbParts * a.n_cb);
+        ld_table_body<T>(a.dt, a.dt_f32, a.dt_bias, a.A, a.ldtab, a.lam, a.seqlen, a.nheads, a.nchunks, a.total_bhc, a.dtsb, a.dtsl, blk - kCbParts * a.n_cb);
     }
 }
 

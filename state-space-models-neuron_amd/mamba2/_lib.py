@@ -46,7 +46,8 @@ class SsdParams(C.Structure):
                 ("ddt_stride_b", _i64), ("ddt_stride_l", _i64),
                 ("dB_stride_b", _i64), ("dB_stride_l", _i64), ("dB_stride_g", _i64),
                 ("dC_stride_b", _i64), ("dC_stride_l", _i64), ("dC_stride_g", _i64),
-                ("dtype", _i32), ("dt_dtype", _i32)]
+                ("dtype", _i32), ("dt_dtype", _i32),
+                ("dt_bias", _vp), ("d_dt_bias", _vp)]
 
 
 class DecodeParams(C.Structure):

@@ -4,7 +4,9 @@
                         n_groups, ssm_state_size, intermediate_size, head_dim) -> norm_out[b,l,d_inner]
 
 Pipeline (``fused_kernel.py:252-282``): split [z | xBC | dt] -> depthwise conv + SiLU ->
-softplus(dt + dt_bias) -> SSD scan -> gated RMSNorm per group (eps 1e-5).
+softplus(dt + dt_bias) -> SSD scan -> gated RMSNorm per group (eps 1e-5).  Here that is three kernel
+stages: conv, scan (softplus applied where the scan builds its decay tables, its gradient and d_dt_bias
+formed where the scan writes ddt), norm.
 
 Every stage is a HIP kernel.  The split is never materialised: the kernels take strided views of ``zxBCdt`` (the conv reads
 the xBC columns in place; the scan reads x, B, C as views of the conv output), and in the backward
@@ -48,17 +50,17 @@ def _forward_parts(zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, n_groups, d
     b, l, _ = zxBCdt.shape
     conv_out = torch.empty((b, l, d_conv), dtype=zxBCdt.dtype, device=zxBCdt.device)
     conv1d_forward(xBC, conv_w, conv_b, "silu", channels_last=True, out=conv_out)
-    dt_sp = glue.softplus_bias_hip(dt, dt_bias)
     x, Bm, Cm = _xbc_views(conv_out, n_groups, d_state, d_inner, d_head)
     # the scan's chunk states are kept for the backward when one follows directly (no second recompute there)
-    states = alloc_chunk_states(dt_sp, logA, x, Bm, Cm) if (keep_states and x.numel() > 0) else None
-    y, _ = ssd_forward(dt_sp, logA, x, Bm, Cm, D, chunk_states=states)
+    states = alloc_chunk_states(dt, logA, x, Bm, Cm) if (keep_states and x.numel() > 0) else None
+    # softplus(dt + dt_bias) is applied inside the scan, on the dt columns of zxBCdt where they lie
+    y, _ = ssd_forward(dt, logA, x, Bm, Cm, D, chunk_states=states, dt_bias=dt_bias)
     scan_out = y.view(b, l, d_inner)
     norm_out = glue.rmsnorm_gated_hip(scan_out, z, norm_w, n_groups, NORM_EPS, out_dtype=zxBCdt.dtype)
-    return norm_out, conv_out, dt_sp, scan_out, states
+    return norm_out, conv_out, scan_out, states
 
 
-def _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out, states,
+def _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, scan_out, states,
                     n_groups, d_state, d_inner, d_head):
     z, xBC, dt, h, d_conv = _views(zxBCdt, n_groups, d_state, d_inner, d_head)
     b, l, width = zxBCdt.shape
@@ -72,10 +74,11 @@ def _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, 
     x, Bm, Cm = _xbc_views(conv_out, n_groups, d_state, d_inner, d_head)
     d_conv_out = torch.empty_like(conv_out)
     dx_v, dB_v, dC_v = _xbc_views(d_conv_out, n_groups, d_state, d_inner, d_head)
-    d_dt_sp, d_logA, _, _, _, d_D, _ = ssd_backward(dt_sp, logA, x, Bm, Cm, D, d_scan_out.view(b, l, h, d_head),
-                                                     out_dX=dx_v, out_dB=dB_v, out_dC=dC_v, chunk_states=states)
-    # softplus backward (into the dt columns) and conv backward (into the xBC columns)
-    _, d_dt_bias = glue.softplus_bias_bwd_hip(dt, dt_bias, d_dt_sp, out_d_in=ddt_view)
+    # (the gradient of the raw dt goes straight into the dt columns of d_zxBCdt, d_dt_bias comes back summed)
+    _, d_logA, _, _, _, d_D, _, d_dt_bias = ssd_backward(dt, logA, x, Bm, Cm, D, d_scan_out.view(b, l, h, d_head),
+                                                         out_dX=dx_v, out_dB=dB_v, out_dC=dC_v, chunk_states=states,
+                                                         dt_bias=dt_bias, out_ddt=ddt_view)
+    # conv backward (into the xBC columns)
     _, d_conv_w, d_conv_b = conv1d_backward(xBC, conv_w, conv_b, d_conv_out, "silu", channels_last=True, out_dx=dxBC_view)
     return (d_zxBCdt, d_logA.to(logA.dtype), d_D.to(D.dtype) if D is not None else None, d_conv_w, d_conv_b,
             d_dt_bias.to(dt_bias.dtype), d_norm_w.to(norm_w.dtype))
@@ -95,10 +98,8 @@ class Mamba2FusedKernel(torch.autograd.Function):
     def backward(ctx, d_output):
         zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w = ctx.saved_tensors
         # recompute conv, softplus and scan (only the inputs were saved)
-        _, conv_out, dt_sp, scan_out, states = _forward_parts(zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, *ctx.dims,
-                                                              keep_states=True)
-        grads = _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out, states,
-                                *ctx.dims)
+        _, conv_out, scan_out, states = _forward_parts(zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, *ctx.dims, keep_states=True)
+        grads = _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, scan_out, states, *ctx.dims)
         return (*grads, None, None, None, None)
 
 
@@ -106,18 +107,18 @@ class Mamba2FusedKernelWithCaching(torch.autograd.Function):
     @staticmethod
     def forward(ctx, zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias,
                 norm_weight, n_groups, ssm_state_size, intermediate_size, head_dim):
-        norm_out, conv_out, dt_sp, scan_out, states = _forward_parts(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias,
-                                                                     norm_weight, n_groups, ssm_state_size, intermediate_size,
-                                                                     head_dim, keep_states=True)
+        norm_out, conv_out, scan_out, states = _forward_parts(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias,
+                                                              norm_weight, n_groups, ssm_state_size, intermediate_size,
+                                                              head_dim, keep_states=True)
         ctx.dims = (n_groups, ssm_state_size, intermediate_size, head_dim)
         ctx.chunk_states = states
-        ctx.save_for_backward(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias, norm_weight, conv_out, dt_sp, scan_out)
+        ctx.save_for_backward(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias, norm_weight, conv_out, scan_out)
         return norm_out
 
     @staticmethod
     def backward(ctx, d_output):
-        zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out = ctx.saved_tensors
-        grads = _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, dt_sp, scan_out,
+        zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, scan_out = ctx.saved_tensors
+        grads = _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, conv_out, scan_out,
                                 ctx.chunk_states, *ctx.dims)
         return (*grads, None, None, None, None)
 

@@ -24,8 +24,9 @@ def _check_inner(name, t):
         raise ValueError(f"{name}: innermost dimension must be contiguous (stride {t.stride(-1)})")
 
 
-def _fill_common(p, dt, A, X, B, C, D):
+def _fill_common(p, dt, A, X, B, C, D, dt_bias=None):
     b, l, h, hd = X.shape
+    p.dt_bias = ptr(dt_bias)
     g, n = B.shape[2], B.shape[3]
     p.x, p.dt, p.A, p.B, p.C, p.D = ptr(X), ptr(dt), ptr(A), ptr(B), ptr(C), ptr(D)
     p.batch, p.seqlen, p.nheads, p.headdim, p.dstate, p.ngroups = b, l, h, hd, n, g
@@ -60,6 +61,15 @@ def _validate(dt, A, X, B, C, D, initial_state):
     _lib.require_gpu(dt, A, X, B, C, D, initial_state)
 
 
+def _bias32(dt_bias, h):
+    if dt_bias is None:
+        return None
+    if dt_bias.shape != (h,):
+        raise ValueError("dt_bias must have shape (n_heads,)")
+    _lib.require_gpu(dt_bias)
+    return dt_bias.detach().float().contiguous()
+
+
 def alloc_chunk_states(dt, A, X, B, C):
     """Carry-over buffer from ``ssd_forward(..., chunk_states=buf)`` to ``ssd_backward(..., chunk_states=buf)``
     (opaque bytes): the SSM state entering each 128-token chunk -- the first b*ceil(l/128)*h*p*n elements, in
@@ -70,8 +80,9 @@ def alloc_chunk_states(dt, A, X, B, C):
     return torch.empty(lib.m2_ssd_chunk_states_bytes(p), dtype=torch.uint8, device=X.device)
 
 
-def ssd_forward(dt, A, X, B, C, D=None, initial_state=None, want_final_state=False, chunk_states=None):
-    """Raw forward through the C ABI.  Returns (Y, final_state or None)."""
+def ssd_forward(dt, A, X, B, C, D=None, initial_state=None, want_final_state=False, chunk_states=None, dt_bias=None):
+    """Raw forward through the C ABI.  Returns (Y, final_state or None).
+    With ``dt_bias`` (h), ``dt`` is the raw projection output and the step size is softplus(dt + dt_bias), applied inside."""
     _validate(dt, A, X, B, C, D, initial_state)
     lib = _lib.load()
     b, l, h, hd = X.shape
@@ -82,7 +93,8 @@ def ssd_forward(dt, A, X, B, C, D=None, initial_state=None, want_final_state=Fal
     Y = torch.empty((b, l, h, hd), dtype=X.dtype, device=X.device)
     S = torch.empty((b, h, hd, n), dtype=torch.float32, device=X.device) if want_final_state else None
     p = SsdParams()
-    _fill_common(p, dt, A32, X, B, C, D32)
+    bias32 = _bias32(dt_bias, h)
+    _fill_common(p, dt, A32, X, B, C, D32, bias32)
     p.initial_state, p.final_state, p.y = ptr(S0), ptr(S), ptr(Y)
     p.chunk_states = _chunk_states_ptr(lib, p, chunk_states)
     p.y_stride_b, p.y_stride_l, p.y_stride_h = _strides3(Y)
@@ -104,10 +116,11 @@ def _chunk_states_ptr(lib, p, chunk_states):
 
 
 def ssd_backward(dt, A, X, B, C, D, dY, initial_state=None, d_final_state=None, want_dinitial=False,
-                 out_dX=None, out_dB=None, out_dC=None, chunk_states=None):
+                 out_dX=None, out_dB=None, out_dC=None, chunk_states=None, dt_bias=None, out_ddt=None):
     """Raw backward through the C ABI.
-    Returns (ddt, dA fp32 (h), dX, dB, dC, dD fp32 (h) or None, d_initial_state or None).
-    ``out_dX/out_dB/out_dC`` let the caller provide (strided) destinations, e.g. views of a packed
+    Returns (ddt, dA fp32 (h), dX, dB, dC, dD fp32 (h) or None, d_initial_state or None), and as an eighth element
+    d_dt_bias fp32 (h) when ``dt_bias`` is given (``dt`` is then the raw projection output and ddt its gradient).
+    ``out_dX/out_dB/out_dC/out_ddt`` let the caller provide (strided) destinations, e.g. views of a packed
     [dx | dB | dC] buffer.  ``chunk_states``: what the forward wrote for the same inputs (skips the recompute)."""
     lib = _lib.load()
     b, l, h, hd = X.shape
@@ -122,7 +135,11 @@ def ssd_backward(dt, A, X, B, C, D, dY, initial_state=None, d_final_state=None, 
     esz = dY.element_size()
     if any((s * esz) % 16 for s in dY.stride()[:3]) or dY.data_ptr() % 16:
         dY = dY.contiguous()
-    ddt = torch.empty((b, l, h), dtype=dt.dtype, device=dev)
+    if out_ddt is not None and (out_ddt.shape != (b, l, h) or out_ddt.dtype != dt.dtype or out_ddt.stride(-1) != 1):
+        raise ValueError("out_ddt must have the shape and dtype of dt, heads contiguous")
+    ddt = out_ddt if out_ddt is not None else torch.empty((b, l, h), dtype=dt.dtype, device=dev)
+    bias32 = _bias32(dt_bias, h)
+    d_bias = torch.empty((h,), dtype=torch.float32, device=dev) if dt_bias is not None else None
     dX = out_dX if out_dX is not None else torch.empty((b, l, h, hd), dtype=X.dtype, device=dev)
     dB = out_dB if out_dB is not None else torch.empty((b, l, g, n), dtype=B.dtype, device=dev)
     dC = out_dC if out_dC is not None else torch.empty((b, l, g, n), dtype=C.dtype, device=dev)
@@ -130,7 +147,8 @@ def ssd_backward(dt, A, X, B, C, D, dY, initial_state=None, d_final_state=None, 
     dD = torch.empty((h,), dtype=torch.float32, device=dev) if D is not None else None
     dS0 = torch.empty((b, h, hd, n), dtype=torch.float32, device=dev) if want_dinitial else None
     p = SsdParams()
-    _fill_common(p, dt, A32, X, B, C, D32)
+    _fill_common(p, dt, A32, X, B, C, D32, bias32)
+    p.d_dt_bias = ptr(d_bias)
     p.initial_state, p.dy, p.d_final_state = ptr(S0), ptr(dY), ptr(dSf)
     p.chunk_states = _chunk_states_ptr(lib, p, chunk_states)
     p.dx, p.ddt, p.dA, p.dB, p.dC, p.dD, p.d_initial_state = ptr(dX), ptr(ddt), ptr(dA), ptr(dB), ptr(dC), ptr(dD), ptr(dS0)
@@ -144,6 +162,8 @@ def ssd_backward(dt, A, X, B, C, D, dY, initial_state=None, d_final_state=None, 
     p.workspace, p.workspace_bytes = ptr(ws), ws.numel()
     with torch.cuda.device(dev):
         _lib.check(lib.m2_ssd_bwd(p, _lib.stream_ptr(dev)), "m2_ssd_bwd")
+    if dt_bias is not None:
+        return ddt, dA, dX, dB, dC, dD, dS0, d_bias
     return ddt, dA, dX, dB, dC, dD, dS0
 
 

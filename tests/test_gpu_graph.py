@@ -74,8 +74,8 @@ def test_fused_core_graph_replay():
 
     def step():
         with torch.no_grad():
-            norm_out, conv_out, dt_sp, scan_out, states = _forward_parts(zx, A, D, cw, cb, dtb, nw, *dims, keep_states=True)
-            grads = _backward_parts(dout, zx, A, D, cw, cb, dtb, nw, conv_out, dt_sp, scan_out, states, *dims)
+            norm_out, conv_out, scan_out, states = _forward_parts(zx, A, D, cw, cb, dtb, nw, *dims, keep_states=True)
+            grads = _backward_parts(dout, zx, A, D, cw, cb, dtb, nw, conv_out, scan_out, states, *dims)
         return (norm_out,) + tuple(grads)
 
     graph, outs = _capture(step)

@@ -177,3 +177,49 @@ def test_ssd_backward_kept_chunk_states_equal_recompute(dtype):
         assert torch.equal(a_, b_)
     with pytest.raises(ValueError, match="chunk_states"):
         ssd_backward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], d["dy"], chunk_states=states[:-256].contiguous())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("b,l,h,p,n,g", [(2, 384, 4, 64, 128, 2), (1, 200, 2, 128, 64, 1), (1, 77, 8, 64, 64, 1)])
+def test_ssd_softplus_folded_into_scan(dtype, b, l, h, p, n, g):
+    """dt_bias given: dt is the raw projection, the step size softplus(dt + dt_bias) is formed inside the scan, the
+    backward returns the gradient of the raw dt and d_dt_bias (fused_kernel.py:33-73, 273, 338)."""
+    from mamba2.mamba2_kernel import alloc_chunk_states, ssd_backward, ssd_forward
+    from oracle.mixer import softplus_ref
+    tol, err = _tol(dtype)
+    d = make_ssd_inputs(b, l, h, p, n, g, seed=l + 7, dtype=dtype)
+    gen = torch.Generator().manual_seed(l)
+    # raw dt as the last h columns of a wider buffer; values on both sides of the softplus threshold
+    raw = (torch.randn(b, l, 24 + h, generator=gen) * 1.5).to(dtype)
+    if dtype == torch.float32:
+        raw[0, : l // 8, 24] = 12.0          # beyond the threshold (in bf16 such steps, 100 x the usual size, only test the error metric)
+    bias = torch.empty(h).uniform_(-4.0, -1.0, generator=gen)
+    r = _f64(d)
+    dt_raw = raw[..., 24:].double().requires_grad_(True)
+    bias_d = bias.double().requires_grad_(True)
+    lv = {k: r[k].clone().requires_grad_(True) for k in ("A", "X", "B", "C", "D")}
+    y_ref, _ = ssd_chunked_ref(softplus_ref(dt_raw + bias_d), lv["A"], lv["X"], lv["B"], lv["C"], lv["D"], chunk=64)
+    y_ref.backward(r["dy"])
+    g_ = _dev(d)
+    rawg = raw.to(DEV)
+    dtv = rawg[..., 24:]
+    st = alloc_chunk_states(dtv, g_["A"], g_["X"], g_["B"], g_["C"])
+    y, _ = ssd_forward(dtv, g_["A"], g_["X"], g_["B"], g_["C"], g_["D"], chunk_states=st, dt_bias=bias.to(DEV))
+    assert err(y.cpu(), y_ref.detach()) < tol
+    gbuf = torch.full((b, l, 24 + h), 5.0, dtype=dtype, device=DEV)
+    for states in (st, None):        # with the forward's tables, and recomputing them (softplus applied again there)
+        ddt, dA, dX, dB, dC, dD, _, dbias = ssd_backward(dtv, g_["A"], g_["X"], g_["B"], g_["C"], g_["D"], g_["dy"], chunk_states=states,
+                                                          dt_bias=bias.to(DEV), out_ddt=gbuf[..., 24:])
+        assert ddt.data_ptr() == gbuf[..., 24:].data_ptr()
+        if dtype == torch.float32:
+            assert err(ddt.cpu(), dt_raw.grad) < tol
+        else:
+            # stored in bf16, and heavy-tailed here (the tokens with step sizes beyond the threshold): a bf16 value just
+            # above a power of two is off by up to 2^-8 of itself from storage alone, which roundings=2 discounts
+            assert rel_rms_err(ddt.cpu(), dt_raw.grad, roundings=2) < tol
+        # a signed sum over all b * l tokens of ddt terms that are each within the tolerance: a few times the element bound
+        assert err(dbias.cpu(), bias_d.grad) < (5e-4 if dtype == torch.float32 else tol)
+        assert err(dX.cpu(), lv["X"].grad) < tol
+        # dA, like d_dt_bias, is a signed sum over all tokens (here with step sizes from 1e-2 up to 11, beyond the threshold)
+        assert err(dA.cpu(), lv["A"].grad) < (5e-4 if dtype == torch.float32 else tol)
+        assert torch.equal(gbuf[..., :24], torch.full((b, l, 24), 5.0, dtype=dtype, device=DEV))
