@@ -2,7 +2,7 @@
 
 * sequence split: scanning the whole sequence == scanning its two halves with the final state of the first handed to
   the second as initial state (forward), for the 2.7B (c1) and 7B-layer (c3) SSD shapes;
-* linearity of the backward in dy, and dD == sum(dy * x) (mamba2_kernel.py:471), at the c1 shape;
+* linearity of the backward in dy, and dD == sum(dy * x) (mamba2_kernel.py:471), at the c1 and c3 shapes;
 * conv: shifting the input by one token shifts the output by one token (causality + time invariance), c2 shape;
 * decode: 4 token steps from the prefill's final state == the chunked scan over the 4 extra tokens, c4 width.
 """
@@ -35,9 +35,9 @@ def test_ssd_sequence_split_bf16(b, l, h, p, n, g):
     assert (S2 - S).norm() / S.norm() < 5e-3
 
 
-def test_ssd_backward_linearity_c1():
+@pytest.mark.parametrize("b,l,h,p,n,g", [(4, 2048, 80, 64, 128, 1), (2, 4096, 128, 64, 128, 8)])
+def test_ssd_backward_linearity(b, l, h, p, n, g):
     from mamba2.mamba2_kernel import alloc_chunk_states, ssd_backward, ssd_forward
-    b, l, h, p, n, g = 4, 2048, 80, 64, 128, 1
     d = make_ssd_inputs(b, l, h, p, n, g, seed=5, dtype=torch.bfloat16, device=DEV)
     st = alloc_chunk_states(d["dt"], d["A"], d["X"], d["B"], d["C"])
     ssd_forward(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], chunk_states=st)
