@@ -98,18 +98,21 @@ dg16_kernel(const T* __restrict__ X, const float* __restrict__ ldtab,
     floatx16 dG = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     // row sums of block (rb, cb) go to rs[cb], column sums to cs[rb]; token t collects rs[0 .. t/32] and cs[t/32 .. 3]
+    // (done by waves 2 and 3, which sit on the SIMDs that carry two waves; all eight values are read and the unwanted
+    // ones dropped by a select: a branch per term costs more than the reads)
     auto flush_sums = [&](int64_t h, int par) {
-        if (tid < kQ) {
+        const int t = tid - 2 * 64;
+        if (t >= 0 && t < kQ) {
             const float* rs = s_sum + par * 8 * kQ;
             const float* cs = rs + 4 * kQ;
-            const int tb = tid >> 5;
+            const int tb = t >> 5;
             float acc = 0.f;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                if (q <= tb) acc += rs[q * kQ + tid];
-                if (q >= tb) acc -= cs[q * kQ + tid];
+                const float rv = rs[q * kQ + t], cv = cs[q * kQ + t];
+                acc += (q <= tb ? rv : 0.f) - (q >= tb ? cv : 0.f);
             }
-            dl_diag[((b * nheads + h) * nchunks + c) * kQ + tid] = acc;
+            dl_diag[((b * nheads + h) * nchunks + c) * kQ + t] = acc;
         }
     };
 
