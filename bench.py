@@ -272,6 +272,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all", choices=["all", "ssd", "conv", "glue", "core", "decode", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--exclude", default="", help="comma-separated workloads to leave out of --workload all (for per-kernel profiles)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the hot path has no collective); run with --gpus 1", file=sys.stderr)
@@ -286,7 +287,12 @@ def main():
 
     out = {}
     other = {}
-    if a.workload in ("all", "ssd"):
+    skip = set(x for x in a.exclude.split(",") if x)
+
+    def wanted(name):
+        return a.workload == name or (a.workload == "all" and name not in skip)
+
+    if wanted("ssd"):
         r = bench_ssd(a.steps, a.warmup)
         out.update({
             "metric": "SSD fwd+bwd tokens/s", "value": r["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1,
@@ -303,15 +309,15 @@ def main():
                              "frac": r["io_bytes"] / (r["ms_event_avg"] * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": SSD_TRAFFIC_BYTES,
                              "traffic_rate": SSD_TRAFFIC_BYTES / (r["ms_event_avg"] * 1e-3) / 1e9, "algorithmic_bytes_per_step": r["io_bytes"]},
         })
-    if a.workload in ("all", "conv"):
+    if wanted("conv"):
         other["conv1d"] = bench_conv(a.steps, a.warmup)
-    if a.workload in ("all", "glue"):
+    if wanted("glue"):
         other["mixer_glue"] = bench_glue(a.steps, a.warmup)
-    if a.workload in ("all", "core"):
+    if wanted("core"):
         other["mixer_core"] = bench_core(a.steps, a.warmup)
-    if a.workload in ("all", "decode"):
+    if wanted("decode"):
         other["decode"] = bench_decode(max(3, a.steps // 4), max(1, a.warmup // 2))
-    if a.workload in ("all", "copy"):
+    if wanted("copy"):
         other["stream_copy"] = bench_copy(a.steps, a.warmup)
     if a.workload not in ("all", "ssd"):
         key = {"conv": "conv1d", "glue": "mixer_glue", "core": "mixer_core", "decode": "decode", "copy": "stream_copy"}[a.workload]
@@ -320,7 +326,7 @@ def main():
         out.setdefault("higher_is_better", True)
     if other:
         out["other"] = other
-    if not a.no_cpu and a.workload in ("all", "ssd"):
+    if not a.no_cpu and wanted("ssd"):
         out["cpu_baseline"] = cpu_baseline_ssd()
     print(json.dumps(out))
 
