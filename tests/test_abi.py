@@ -32,7 +32,8 @@ def test_struct_sizes_match_header():
     from mamba2 import _lib
     txt = open(os.path.join(ROOT, "include", "mamba2_hip.h")).read()
     txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
-    for cname, pyc in (("m2_conv1d_params", _lib.Conv1dParams), ("m2_ssd_params", _lib.SsdParams), ("m2_decode_params", _lib.DecodeParams)):
+    for cname, pyc in (("m2_conv1d_params", _lib.Conv1dParams), ("m2_ssd_params", _lib.SsdParams), ("m2_decode_params", _lib.DecodeParams),
+                       ("m2_rmsnorm_params", _lib.RmsnormParams)):
         body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cname, cname), txt, flags=re.S).group(1)
         names = []
         for decl in body.split(";"):
@@ -72,6 +73,23 @@ def test_validation_before_any_device_call(lib):
     assert fw >= tiles * 2 and bw >= fw + tiles * 2      # bf16: the states entering the chunks (+ their gradients)
     s.dtype = 0
     assert lib.m2_ssd_fwd_workspace_bytes(ctypes.byref(s)) >= tiles * 8      # fp32: per-chunk contributions and states
+    # mixer glue
+    n = _lib.RmsnormParams()
+    n.rows, n.channels, n.n_groups, n.dtype = 4, 96, 5, 1
+    assert lib.m2_rmsnorm_gated_fwd(ctypes.byref(n), None) == -1             # channels not divisible by the groups
+    n.n_groups = 8
+    assert lib.m2_rmsnorm_gated_fwd(ctypes.byref(n), None) == -1 and b"multiple of 8" in lib.m2_last_error()
+    n.channels, n.n_groups = 128, 2
+    assert lib.m2_rmsnorm_gated_fwd(ctypes.byref(n), None) == -6             # NULL tensors
+    assert lib.m2_rmsnorm_gated_bwd(ctypes.byref(n), None) == -6
+    n.dtype = 5
+    assert lib.m2_rmsnorm_gated_fwd(ctypes.byref(n), None) == -2
+    assert lib.m2_softplus_bias_fwd(None, 8, None, None, 8, 4, 0, 1, None) == -1      # no heads
+    assert lib.m2_softplus_bias_fwd(None, 8, None, None, 8, 4, 8, 1, None) == -6
+    assert lib.m2_softplus_bias_fwd(None, 8, None, None, 8, 0, 8, 1, None) == 0       # no rows: nothing to do
+    # one partial row of dw per workgroup of the backward (up to one per wave), one partial row of d_bias per 16 rows
+    assert lib.m2_rmsnorm_gated_bwd_workspace_bytes(8192, 5120, 1, 1) >= 512 * 5120 * 4
+    assert lib.m2_softplus_bias_bwd_workspace_bytes(8192, 80) >= (8192 // 16) * 80 * 4
 
 
 def test_python_layer_has_no_cpu_fallback():
@@ -83,6 +101,11 @@ def test_python_layer_has_no_cpu_fallback():
     with pytest.raises(RuntimeError, match="no CPU path"):
         mamba2_kernel(torch.zeros(1, 128, 2), torch.zeros(2), torch.zeros(1, 128, 2, 64), torch.zeros(1, 128, 1, 64),
                       torch.zeros(1, 128, 1, 64), torch.zeros(2))
+    from mamba2 import glue
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        glue.rmsnorm_gated_hip(torch.zeros(2, 64), None, torch.ones(64), 1, 1e-5)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        glue.softplus_bias_hip(torch.zeros(2, 3, 8), torch.zeros(8))
     with pytest.raises(RuntimeError, match="no CPU path"):
         mamba2_kernel_inference(torch.zeros(1, 1, 40), torch.zeros(1, 40, 3), torch.zeros(40, 4), torch.zeros(40),
                                 torch.zeros(1, 2, 4, 16), torch.zeros(1, 1, 2), torch.zeros(2), torch.zeros(2))
