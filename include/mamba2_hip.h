@@ -154,6 +154,9 @@ typedef struct m2_decode_params {
     int32_t dtype;                                      /* xBC, conv_state, dt, y       */
     int32_t param_dtype;                                /* conv_w, conv_b               */
     int32_t activation;
+    const float* dt_bias;                               /* (h) or NULL.  Given: dt holds the raw projection output and the
+                                                           step size is softplus(dt + dt_bias), threshold form
+                                                           (mamba2/mamba2_mixer.py:268), applied inside in fp32            */
 } m2_decode_params;
 
 size_t m2_decode_workspace_bytes(int64_t batch, int64_t nheads, int64_t headdim, int64_t dstate, int64_t ngroups);

@@ -68,7 +68,7 @@ __global__ void __launch_bounds__(256) stream_copy_kernel(const uint4* __restric
 }  // namespace
 }  // namespace m2
 
-extern "C" int m2_abi_version(void) { return 2; }
+extern "C" int m2_abi_version(void) { return 3; }
 extern "C" const char* m2_last_error(void) { return m2::g_err; }
 
 extern "C" int m2_mfma_selftest(const void* A, const void* Bt, float* C, int64_t M, int64_t N, int64_t K, int32_t dtype, void* stream) {

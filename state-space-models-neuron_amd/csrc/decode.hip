@@ -125,8 +125,8 @@ __device__ __forceinline__ float group_sum(float v, int GL) {
 template <typename T, int VEC>
 __global__ void __launch_bounds__(256)
 decode_ssm_kernel(float* __restrict__ S, const float* __restrict__ act, const T* __restrict__ dt, const float* __restrict__ A,
-                  const float* __restrict__ D, T* __restrict__ y, int64_t nheads, int P, int N, int64_t ngroups, int64_t Cx,
-                  int64_t dtsb, int64_t ysb, int GL) {
+                  const float* __restrict__ D, const float* __restrict__ dt_bias, T* __restrict__ y, int64_t nheads, int P, int N,
+                  int64_t ngroups, int64_t Cx, int64_t dtsb, int64_t ysb, int GL) {
     const int tid = threadIdx.x;
     const int64_t h = blockIdx.x, b = blockIdx.y;
     const int64_t g = h / (nheads / ngroups);
@@ -134,7 +134,9 @@ decode_ssm_kernel(float* __restrict__ S, const float* __restrict__ act, const T*
     const float* xa = act + b * Cx + h * P;
     const float* Ba = act + b * Cx + d_inner + g * N;
     const float* Ca = act + b * Cx + d_inner + ngroups * N + g * N;
-    const float dtv = to_f32(dt[b * dtsb + h]);
+    // with dt_bias, dt is the raw projection output and the step size is softplus(dt + dt_bias)  (mamba2_mixer.py:268)
+    float dtv = to_f32(dt[b * dtsb + h]);
+    if (dt_bias) dtv = softplus_f(dtv + dt_bias[h]);
     const float dA = __expf(A[h] * dtv);
     const float Dh = D ? D[h] : 0.f;
     float* Sp = S + (b * nheads + h) * (int64_t)P * N;
@@ -253,10 +255,10 @@ extern "C" int m2_decode_step(const m2_decode_params* p, void* stream) {
         if (rc2) return rc2;
         dim3 grid((unsigned)p->nheads, (unsigned)p->batch);
         if (vec == 4)
-            decode_ssm_kernel<T, 4><<<grid, 256, 0, st>>>(p->S, act, static_cast<const T*>(p->dt), p->A, p->D, static_cast<T*>(p->y),
+            decode_ssm_kernel<T, 4><<<grid, 256, 0, st>>>(p->S, act, static_cast<const T*>(p->dt), p->A, p->D, p->dt_bias, static_cast<T*>(p->y),
                                                           p->nheads, (int)p->headdim, (int)p->dstate, p->ngroups, Cx, p->dt_stride_b, p->y_stride_b, GL);
         else
-            decode_ssm_kernel<T, 1><<<grid, 256, 0, st>>>(p->S, act, static_cast<const T*>(p->dt), p->A, p->D, static_cast<T*>(p->y),
+            decode_ssm_kernel<T, 1><<<grid, 256, 0, st>>>(p->S, act, static_cast<const T*>(p->dt), p->A, p->D, p->dt_bias, static_cast<T*>(p->y),
                                                           p->nheads, (int)p->headdim, (int)p->dstate, p->ngroups, Cx, p->dt_stride_b, p->y_stride_b, GL);
         return check_launch("decode_ssm_kernel");
     });

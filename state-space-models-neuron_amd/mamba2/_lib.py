@@ -57,7 +57,7 @@ class DecodeParams(C.Structure):
                 ("batch", _i64), ("nheads", _i64), ("headdim", _i64), ("dstate", _i64), ("ngroups", _i64),
                 ("k", _i32), ("W", _i32),
                 ("xBC_stride_b", _i64), ("dt_stride_b", _i64), ("y_stride_b", _i64),
-                ("dtype", _i32), ("param_dtype", _i32), ("activation", _i32)]
+                ("dtype", _i32), ("param_dtype", _i32), ("activation", _i32), ("dt_bias", _vp)]
 
 
 class RmsnormParams(C.Structure):

@@ -14,6 +14,11 @@ the scan writes dx, dB, dC straight into one packed buffer and the conv writes i
 the xBC columns of ``d_zxBCdt``.  ``Mamba2FusedKernel`` saves only its inputs and recomputes conv,
 softplus and scan in the backward (as the reference does, ``:352-367``); ``...WithCaching`` keeps the
 intermediates (``:449-471``).
+
+``mamba2_fused_prefill`` is the inference form of the same pipeline that also hands the sequence over to the
+decode step: it leaves the SSM state after the last token and the last W conv inputs in the caller's cache
+tensors, and continues from them when the cache already holds a prefix.  The reference has no such path
+(``mamba2_mixer.py:220``: "cache not supported yet"); the layouts are those its ``step`` reads (``:270-276``).
 """
 import torch
 
@@ -137,3 +142,37 @@ def mamba2_fused_kernel_with_caching(zxBCdt, logA, D, conv1d_weight, conv1d_bias
     return Mamba2FusedKernelWithCaching.apply(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias,
                                               norm_weight, n_groups, ssm_state_size, intermediate_size,
                                               head_dim)
+
+
+def mamba2_fused_prefill(zxBCdt, logA, D, conv1d_weight, conv1d_bias, dt_bias, norm_weight, n_groups, ssm_state_size,
+                         intermediate_size, head_dim, conv_state, ssm_state, continuing=False):
+    """Inference forward ``zxBCdt -> norm_out`` that updates the decode cache in place.
+
+    ``conv_state`` (b, conv_dim, W), W in {k-1, k}: on return the last W rows of xBC (before the conv), oldest first.
+    ``ssm_state`` (b, h, p, n) fp32: on return the scan's state after the last token.
+    ``continuing``: the two tensors hold the state after an earlier prefix (prefill in pieces, or prefill after decode
+    steps); otherwise they are taken as zero and only written."""
+    z, xBC, dt, h, d_conv = _views(zxBCdt, n_groups, ssm_state_size, intermediate_size, head_dim)
+    b, l, _ = zxBCdt.shape
+    k, W = conv1d_weight.shape[-1], conv_state.shape[-1]
+    if conv_state.shape != (b, d_conv, W) or not (k - 1 <= W):
+        raise ValueError(f"conv_state must be (b, conv_dim, W >= k-1), got {tuple(conv_state.shape)}")
+    if ssm_state.shape != (b, h, head_dim, ssm_state_size) or ssm_state.dtype != torch.float32:
+        raise ValueError("ssm_state must be (b, h, p, n) float32")
+    if l == 0:
+        return torch.empty((b, 0, intermediate_size), dtype=zxBCdt.dtype, device=zxBCdt.device)
+    with torch.no_grad():
+        if continuing:
+            # the cached inputs go in front of the new ones; the outputs for them are dropped
+            hist = torch.cat([conv_state.transpose(1, 2).to(xBC.dtype), xBC], dim=1)
+            conv_out = conv1d_forward(hist, conv1d_weight, conv1d_bias, "silu", channels_last=True)[:, W:]
+            tail = hist[:, l:]
+        else:
+            conv_out = conv1d_forward(xBC, conv1d_weight, conv1d_bias, "silu", channels_last=True)
+            tail = xBC[:, l - W:] if l >= W else torch.cat([xBC.new_zeros(b, W - l, d_conv), xBC], dim=1)
+        x, Bm, Cm = _xbc_views(conv_out, n_groups, ssm_state_size, intermediate_size, head_dim)
+        y, S = ssd_forward(dt, logA, x, Bm, Cm, D, initial_state=ssm_state if continuing else None, want_final_state=True,
+                           dt_bias=dt_bias)
+        ssm_state.copy_(S)
+        conv_state.copy_(tail.transpose(1, 2))
+        return glue.rmsnorm_gated_hip(y.view(b, l, intermediate_size), z, norm_weight, n_groups, NORM_EPS, out_dtype=zxBCdt.dtype)

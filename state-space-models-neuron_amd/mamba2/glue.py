@@ -1,9 +1,10 @@
 """Elementwise glue of the mixer core: softplus(dt + dt_bias) and the gated, grouped RMSNorm, forward and
 backward (``mamba2/fused_kernel.py:33-73,76-175``; torch twins ``mamba2/mamba2_mixer.py:36-38,88-105``).
 
-Two forms.  The ``*_hip`` functions call the HIP kernels (one pass over each tensor, strided rows taken in place) and
-are what the fused mixer core uses.  The plain functions are the same math as differentiable torch device ops, for
-``MambaRMSNormGated`` used as an ordinary module (autograd builds its backward) and for the one-token decode step.
+Three forms.  The ``*_hip`` functions call the HIP kernels (one pass over each tensor, strided rows taken in place) and
+are what the fused mixer core uses.  ``rmsnorm_gated_fn`` wraps the forward and backward kernels in an autograd function,
+for the norm modules (``MambaRMSNormGated``, the blocks' ``Mamba2RMSNorm``) and the one-token decode step.  The plain
+functions are the same math as differentiable torch device ops, for group widths the kernels do not hold in registers.
 """
 import ctypes as C
 
@@ -192,3 +193,38 @@ def rmsnorm_gated_bwd_hip(x, z, weight, d_out, n_groups, eps, out_dz=None):
         out_dz.copy_(dz)
         dz = out_dz
     return dx, dw, dz
+
+
+# --------------------------------------------------------------------------------------------- autograd form
+def norm_kernel_ok(x, n_groups):
+    """True if the HIP norm kernels take this shape: group width a multiple of the vector width and within a row's registers."""
+    if x.dtype not in (torch.float32, torch.bfloat16) or n_groups < 1 or x.shape[-1] % n_groups:
+        return False
+    gw = x.shape[-1] // n_groups
+    vec, cap = (8, 8192) if x.dtype == torch.bfloat16 else (4, 4096)
+    return gw % vec == 0 and 0 < gw <= cap
+
+
+class RmsnormGated(torch.autograd.Function):
+    """Gated grouped RMSNorm on the HIP kernels, forward and backward (z may be None: plain RMSNorm)."""
+
+    @staticmethod
+    def forward(ctx, x, z, weight, n_groups, eps, out_dtype):
+        ctx.save_for_backward(x, z, weight)
+        ctx.n_groups, ctx.eps = n_groups, eps
+        return rmsnorm_gated_hip(x, z, weight, n_groups, eps, out_dtype=out_dtype)
+
+    @staticmethod
+    def backward(ctx, d_out):
+        x, z, weight = ctx.saved_tensors
+        dx, dw, dz = rmsnorm_gated_bwd_hip(x, z, weight, d_out, ctx.n_groups, ctx.eps)
+        return dx, dz, dw.to(weight.dtype), None, None, None
+
+
+def rmsnorm_gated_fn(x, z, weight, n_groups, eps, out_dtype=None):
+    """Differentiable gated grouped RMSNorm; output fp32 unless ``out_dtype`` says the dtype of x.
+    Shapes outside the kernels' limits go through the torch device ops (same math, autograd builds the backward)."""
+    _lib.require_gpu(x, z, weight)
+    if not norm_kernel_ok(x, n_groups) or (z is not None and z.dtype != x.dtype):
+        return rmsnorm_gated(x, z, weight, n_groups, eps, out_dtype=out_dtype)
+    return RmsnormGated.apply(x, z, weight, n_groups, eps, out_dtype)

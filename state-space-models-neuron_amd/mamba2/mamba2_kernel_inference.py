@@ -8,7 +8,9 @@
 Unlike the reference, which writes fresh output tensors, ``conv_state`` and ``S`` are updated IN
 PLACE and the same tensors are returned, which is compatible with the caller's re-binding of the
 cache entries (``mamba2/mamba2_mixer.py:275-276``).  W may be k-1 or k columns.  The SSM state must
-be float32.
+be float32.  ``xBC`` and ``dt`` may be column slices of the packed projection output.  With the keyword
+``dt_bias`` (h), ``dt`` is the raw projection output and the kernel applies softplus(dt + dt_bias) itself
+(the caller's ``softplus`` pass of ``mamba2_mixer.py:268`` is then not needed).
 """
 import torch
 
@@ -17,7 +19,7 @@ from ._lib import DecodeParams, ptr
 
 
 def mamba2_kernel_inference(xBC_tensor, conv_state_tensor, conv_weight_tensor, conv_bias_tensor, S_tensor, dt_tensor,
-                            logA_tensor, D_tensor=None, n_groups=1, activation="silu"):
+                            logA_tensor, D_tensor=None, n_groups=1, activation="silu", dt_bias=None):
     batch_size, n_heads, d_head, d_state = S_tensor.shape
     seq_len = xBC_tensor.shape[1]
     assert seq_len == 1
@@ -36,13 +38,17 @@ def mamba2_kernel_inference(xBC_tensor, conv_state_tensor, conv_weight_tensor, c
         raise ValueError("S and conv_state must be contiguous (they are updated in place)")
     if xBC_tensor.stride(-1) != 1 or dt_tensor.stride(-1) != 1:
         raise ValueError("xBC and dt must be contiguous in their last dimension")
-    _lib.require_gpu(xBC_tensor, conv_state_tensor, conv_weight_tensor, conv_bias_tensor, S_tensor, dt_tensor, logA_tensor, D_tensor)
+    _lib.require_gpu(xBC_tensor, conv_state_tensor, conv_weight_tensor, conv_bias_tensor, S_tensor, dt_tensor, logA_tensor, D_tensor,
+                     dt_bias)
+    if dt_bias is not None and dt_bias.shape != (n_heads,):
+        raise ValueError("dt_bias must have shape (n_heads,)")
     lib = _lib.load()
     dev = xBC_tensor.device
     w = conv_weight_tensor.detach().reshape(d_xBC, k).contiguous()
     bias = conv_bias_tensor.detach().contiguous() if conv_bias_tensor is not None else None
     A32 = logA_tensor.detach().float().contiguous()
     D32 = D_tensor.detach().float().contiguous() if D_tensor is not None else None
+    bias32 = dt_bias.detach().float().contiguous() if dt_bias is not None else None
     out_Y = torch.empty((batch_size, seq_len, d_inner), device=dev, dtype=xBC_tensor.dtype)
     nbytes = lib.m2_decode_workspace_bytes(batch_size, n_heads, d_head, d_state, n_groups)
     ws = _lib.Workspace.get(nbytes, dev)
@@ -55,6 +61,7 @@ def mamba2_kernel_inference(xBC_tensor, conv_state_tensor, conv_weight_tensor, c
     p.xBC_stride_b, p.dt_stride_b, p.y_stride_b = xBC_tensor.stride(0), dt_tensor.stride(0), out_Y.stride(0)
     p.dtype, p.param_dtype = _lib.dtype_code(xBC_tensor.dtype), _lib.dtype_code(w.dtype)
     p.activation = _lib.ACT[activation]
+    p.dt_bias = ptr(bias32)
     with torch.cuda.device(dev):
         _lib.check(lib.m2_decode_step(p, _lib.stream_ptr(dev)), "m2_decode_step")
     return out_Y, conv_state_tensor, S_tensor

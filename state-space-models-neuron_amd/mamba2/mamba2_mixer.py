@@ -3,8 +3,12 @@
 Parameter names and shapes are the reference's (and HF / state-spaces'): ``in_proj``, ``conv1d.weight (C,1,k)``,
 ``conv1d.bias``, ``dt_bias``, ``A_log``, ``D``, ``norm.weight``, ``out_proj``.  The tensor-parallel linears of the
 reference become ``nn.Linear`` (tp = 1) and its XLA-device assert is dropped.  ``forward`` = in_proj ->
-``mamba2_fused_kernel`` -> out_proj; ``step`` = in_proj -> split -> softplus -> ``mamba2_kernel_inference`` ->
-gated norm -> out_proj.
+``mamba2_fused_kernel`` -> out_proj; ``step`` = in_proj -> ``mamba2_kernel_inference`` on the [xBC | dt] columns
+(softplus applied inside) -> gated norm -> out_proj: two projections and three kernels of this library per token.
+
+``forward`` with ``cache_params`` (inference only) is the prefill that hands over to ``step``: it leaves the layer's
+SSM and conv state in the cache, and continues from them when ``cache_params.seqlen_offset > 0``.  The reference
+asserts the cache away there (``mamba2_mixer.py:220``); the cache fields are the ones its ``step`` uses (``:270-276``).
 """
 import math
 from typing import Optional
@@ -14,7 +18,7 @@ from torch import nn
 
 from .configuration_mamba2 import Mamba2Config
 from .conv1d_grouped import ConvNKI
-from .fused_kernel import mamba2_fused_kernel
+from .fused_kernel import mamba2_fused_kernel, mamba2_fused_prefill
 from .mamba2_kernel_inference import mamba2_kernel_inference
 from . import glue
 
@@ -57,9 +61,9 @@ class MambaRMSNormGated(nn.Module):
         self.name = name
         self.hidden_size = hidden_size
 
-    def forward(self, hidden_states, gate=None):
+    def forward(self, hidden_states, gate=None, out_dtype=None):
         g = self.n_groups if self.rmsnorm_within_groups else 1
-        return glue.rmsnorm_gated(hidden_states, gate, self.weight, g, self.eps)
+        return glue.rmsnorm_gated_fn(hidden_states, gate, self.weight, g, self.eps, out_dtype=out_dtype)
 
 
 class Mamba2Mixer(nn.Module):
@@ -122,15 +126,33 @@ class Mamba2Mixer(nn.Module):
         self.n_groups_tp = self.n_groups
         self.num_heads_tp = self.num_heads
         self.conv_dim_tp = self.conv_dim
+        self._fp32_params = None
+
+    def _inference_params(self):
+        """fp32 (A, D, dt_bias) as the decode kernel takes them, rebuilt only when a parameter changed."""
+        ps = (self.A_log, self.D, self.dt_bias)
+        key = tuple((p.data_ptr(), p._version, p.dtype) for p in ps)
+        if self._fp32_params is None or self._fp32_params[0] != key:
+            with torch.no_grad():
+                self._fp32_params = (key, -torch.exp(self.A_log.float()), self.D.float(), self.dt_bias.float())
+        return self._fp32_params[1:]
 
     def nki_kernels_forward(self, hidden_states, cache_params: Optional[Mamba2Cache] = None,
                             cache_position: Optional[torch.LongTensor] = None, attention_mask: Optional[torch.Tensor] = None):
-        assert cache_params is None, "cache not supported yet"
         assert attention_mask is None, "attention mask not supported yet"
         assert self.time_step_limit[0] == 0.0 and self.time_step_limit[1] == float("inf"), "dt limit not supported yet"
         assert self.activation in ["silu", "swish"]
         assert self.rmsnorm_within_groups, "the fused core always normalises within groups (fused_kernel.py:255)"
 
+        if cache_params is not None:
+            assert not torch.is_grad_enabled(), "forward with a cache is the inference prefill: call it under torch.no_grad()"
+            A, D, dt_bias = self._inference_params()
+            zxBCdt = self.in_proj(hidden_states)
+            scan_output = mamba2_fused_prefill(zxBCdt, A, D, self.conv1d.weight, self.conv1d.bias, dt_bias, self.norm.weight,
+                                               self.n_groups_tp, self.ssm_state_size, self.intermediate_size_tp, self.head_dim,
+                                               cache_params.conv_states[self.layer_idx], cache_params.ssm_states[self.layer_idx],
+                                               continuing=cache_params.seqlen_offset > 0)
+            return self.out_proj(scan_output)
         A = -torch.exp(self.A_log.float())
         zxBCdt = self.in_proj(hidden_states)
         scan_output = mamba2_fused_kernel(zxBCdt, A, self.D, self.conv1d.weight, self.conv1d.bias, self.dt_bias, self.norm.weight,
@@ -150,14 +172,13 @@ class Mamba2Mixer(nn.Module):
         n_heads = d_inner // d_head
         d_conv = d_inner + 2 * n_groups * d_state
         assert zxBCdt.shape[-1] == d_inner + d_conv + n_heads
+        # the kernels read the [z | xBC | dt] columns where the projection left them; softplus(dt + dt_bias) happens inside
         z, xBC, dt = torch.split(zxBCdt, [d_inner, d_conv, n_heads], dim=-1)
-        dt = softplus(dt + self.dt_bias).to(xBC.dtype)
-        A = -torch.exp(self.A_log.float())
+        A, D, dt_bias = self._inference_params()
         y, new_conv_state, new_ssm_state = mamba2_kernel_inference(
             xBC, cache_params.conv_states[self.layer_idx], self.conv1d.weight.squeeze(1), self.conv1d.bias,
-            cache_params.ssm_states[self.layer_idx], dt, A, self.D, n_groups=self.n_groups_tp)
+            cache_params.ssm_states[self.layer_idx], dt, A, D, n_groups=self.n_groups_tp, dt_bias=dt_bias)
         cache_params.conv_states[self.layer_idx] = new_conv_state
         cache_params.ssm_states[self.layer_idx] = new_ssm_state
-        y = y.view(batch, seqlen, -1)
-        y = self.norm(y, z).to(hidden_states.dtype)
+        y = self.norm(y.view(batch, seqlen, -1), z, out_dtype=hidden_states.dtype)
         return self.out_proj(y)

@@ -24,7 +24,7 @@ def test_header_symbols_exported_and_bound(lib):
         assert hasattr(lib, s), f"{s} declared in the header but not exported"
         assert s in _lib.SYMBOLS, f"{s} has no ctypes prototype"
     assert sorted(_lib.SYMBOLS) == syms
-    assert lib.m2_abi_version() == 2
+    assert lib.m2_abi_version() == 3
 
 
 def test_struct_sizes_match_header():
