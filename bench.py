@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X Mamba-2 mixer hot path.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|ssd|conv|decode|copy] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|ssd|conv|glue|core|decode|model|copy] [--no-cpu]
 
 One "step" is one pass of the hot path over one batch of synthetic input, inputs resident in HBM:
   ssd    : SSD chunked scan fwd+bwd, bf16, 2.7B shape (b4, l2048, h80, p64, n128, g1, chunk 128)   <- headline
@@ -219,6 +219,47 @@ def bench_decode(steps, warmup):
                           "algorithmic_bytes_per_step": bytes_, "kernels": "decode_conv_kernel + decode_ssm_kernel, 64 launches each"})
 
 
+def bench_model_step(steps, warmup):
+    """One decode step of the whole 2.7B-shaped model (embedding, 64 x [RMSNorm, in_proj, decode kernels, gated norm,
+    out_proj, residual], final norm, LM head) at batch 128: eager launches and the same step replayed from one HIP graph."""
+    import torch
+    from mamba2.configuration_mamba2 import Mamba2Config
+    from mamba2.mamba2_mixer import Mamba2Cache
+    from mamba2.modeling_mamba2 import GraphedStep, Mamba2ForCausalLM
+    cfg = Mamba2Config(num_heads=80, head_dim=64, hidden_size=2560, state_size=128, n_groups=1, num_hidden_layers=64, expand=2,
+                       vocab_size=50288, residual_in_fp32=True)
+    b = DEC_CFG["b"]
+    torch.manual_seed(0)
+    with torch.device("cuda:0"):
+        model = Mamba2ForCausalLM(cfg).to(torch.bfloat16).eval()
+    n_params = sum(p.numel() for p in model.parameters())
+    cache = Mamba2Cache(cfg, b, dtype=torch.bfloat16, device="cuda:0", conv_width=DEC_CFG["W"])
+    gen = torch.Generator(device="cuda:0").manual_seed(0)
+    for t in cache.ssm_states:
+        t.normal_(0.0, 0.1, generator=gen)
+    ids = torch.randint(0, cfg.vocab_size, (b, 1), device="cuda:0", generator=gen)
+
+    def eager():
+        with torch.no_grad():
+            model.step(ids, cache)
+
+    wall_e, per_e = event_time_ms(eager, steps, warmup)
+    graphed = GraphedStep(model, cache, b)
+    wall_g, per_g = event_time_ms(lambda: graphed(ids), steps, warmup)
+    ms_e, ms_g = sum(per_e) / len(per_e), sum(per_g) / len(per_g)
+    # bytes a step has to move: every layer's states read and written, every weight but the embedding table read once
+    state_bytes = sum(2 * t.numel() * t.element_size() for t in cache.ssm_states + cache.conv_states)
+    weight_bytes = (n_params - model.backbone.embeddings.weight.numel()) * 2
+    bytes_ = state_bytes + weight_bytes
+    return dict(metric="whole-model decode step latency (2.7B shape, 64 layers, batch 128), HIP graph", value=ms_g * 1e3, unit="us/step",
+                higher_is_better=False, ms_per_step=ms_g, ms_per_step_eager=ms_e, wall_ms_per_step=wall_g, wall_ms_per_step_eager=wall_e,
+                tokens_per_s=b / (ms_g * 1e-3), parameters=n_params, dtype="bf16 weights and activations / f32 state and residual",
+                config={"workload": "Mamba2ForCausalLM.step, d_model 2560, 64 layers, h80 p64 n128 g1, vocab 50288, b128, conv state W3"},
+                roofline={"bound": "hbm", "achieved": bytes_ / (ms_g * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": bytes_ / (ms_g * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_step": bytes_,
+                          "kernels": "one graph replay: hipBLASLt projections + decode_conv/decode_ssm/rmsnorm_gated kernels + torch elementwise"})
+
+
 def bench_copy(steps, warmup):
     """Plain 16-byte-per-lane copy kernel over 1 GiB (read 1 GiB + write 1 GiB per launch): the HBM rate a trivial
     streaming kernel reaches on this box, and the dispatch of known size the HBM-traffic counters are scaled by."""
@@ -270,7 +311,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", choices=["all", "ssd", "conv", "glue", "core", "decode", "copy"])
+    ap.add_argument("--workload", default="all", choices=["all", "ssd", "conv", "glue", "core", "decode", "model", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--exclude", default="", help="comma-separated workloads to leave out of --workload all (for per-kernel profiles)")
     a = ap.parse_args()
@@ -327,10 +368,12 @@ def main():
         secondary("mixer_core", bench_core, a.steps, a.warmup)
     if wanted("decode"):
         secondary("decode", bench_decode, max(3, a.steps // 4), max(1, a.warmup // 2))
+    if wanted("model"):
+        secondary("decode_model", bench_model_step, max(3, a.steps // 4), max(1, a.warmup // 2))
     if wanted("copy"):
         secondary("stream_copy", bench_copy, a.steps, a.warmup)
     if a.workload not in ("all", "ssd"):
-        key = {"conv": "conv1d", "glue": "mixer_glue", "core": "mixer_core", "decode": "decode", "copy": "stream_copy"}[a.workload]
+        key = {"conv": "conv1d", "glue": "mixer_glue", "core": "mixer_core", "decode": "decode", "model": "decode_model", "copy": "stream_copy"}[a.workload]
         out.update(other.pop(key))
         out.update({"n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "scaling": "weak", "vs_baseline": None, "data": "synthetic"})
         out.setdefault("higher_is_better", True)

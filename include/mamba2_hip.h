@@ -204,6 +204,16 @@ int m2_rmsnorm_gated_fwd(const m2_rmsnorm_params* p, void* stream);
 size_t m2_rmsnorm_gated_bwd_workspace_bytes(int64_t rows, int64_t channels, int32_t n_groups, int32_t dtype);
 int m2_rmsnorm_gated_bwd(const m2_rmsnorm_params* p, void* stream);
 
+/* Block boundary of the token-by-token loop (mamba2/modeling_mamba2.py:133-140 Mamba2Block.step's residual add,
+ * followed by the next block's -- or the final -- Mamba2RMSNorm, :94-103), in one pass over the rows:
+ *   residual += delta;   out = weight * residual * rsqrt(mean(residual^2) + eps)
+ * residual (rows, channels) fp32, updated in place (the fp32 residual stream, residual_in_fp32);
+ * delta (rows, channels) in `dtype`, or NULL (nothing to add: first block); out (rows, channels) in `dtype`; weight fp32.
+ * channels: a multiple of 4, at most 8192.  Inference only (no backward). */
+int m2_add_rmsnorm(float* residual, int64_t residual_stride_row, const void* delta, int64_t delta_stride_row,
+                   const float* weight, void* out, int64_t out_stride_row, int64_t rows, int64_t channels, float eps,
+                   int32_t dtype, void* stream);
+
 /* ------------------------------------------------------------------ self tests / probes
  * m2_mfma_selftest: C (M x N fp32, row-major) = A (M x K) * Bt (N x K)^T through the same
  * LDS-staged MFMA tile code the SSD kernels use.  M, N multiples of 128; K multiple of 32.

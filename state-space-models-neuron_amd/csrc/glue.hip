@@ -279,6 +279,11 @@ int64_t norm_rows_per_block(int64_t rows, int64_t groups, bool bwd) {
     if (rb < 4) rb = 4;
     return (rb + 3) / 4 * 4;
 }
+// the forward with four waves per (row, group) takes one row per pass: few rows (a decode step) spread over more workgroups
+int64_t norm_rows_per_block_fwd(int64_t rows, int64_t groups, int64_t nvec) {
+    if (nvec > 256 && rows * groups < 4096) return 1;
+    return norm_rows_per_block(rows, groups, false);
+}
 // waves per (row, group) and vectors per lane for a group of `nvec` 16-byte vectors; false if it does not fit
 bool norm_shape(int64_t nvec, int* wpg, int* nv) {
     if (nvec <= 0) return false;
@@ -299,6 +304,67 @@ int launch_norm(const NormArgs& a, int64_t groups, hipStream_t st) {
     M2_NORM_CASE(4, 2) M2_NORM_CASE(4, 3) M2_NORM_CASE(4, 4)
 #undef M2_NORM_CASE
     return fail(M2_ERR_SHAPE, "rmsnorm_gated: no kernel for %d waves x %d vectors", wpg, nv);
+}
+
+// Block boundary of a decode step: residual += delta; out = weight * residual * rsqrt(mean(residual^2) + eps).
+// One workgroup per row, the row (up to 8192 channels) stays in registers between the sum of squares and the output.
+template <typename T>
+__global__ void __launch_bounds__(256)
+add_rmsnorm_kernel(float* __restrict__ res, int64_t res_sr, const T* __restrict__ delta, int64_t delta_sr, const float* __restrict__ w,
+                   T* __restrict__ out, int64_t out_sr, int d, float eps) {
+    constexpr int NV = 8;
+    __shared__ float red[4];
+    const int tid = threadIdx.x;
+    const int64_t row = blockIdx.x;
+    float* rr = res + row * res_sr;
+    const T* dr = delta ? delta + row * delta_sr : nullptr;
+    T* orow = out + row * out_sr;
+    const int nvec = d / 4;
+    floatx4 v[NV];
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+        const int vi = it * 256 + tid;
+        v[it] = floatx4{0.f, 0.f, 0.f, 0.f};
+        if (vi < nvec) {
+            floatx4 r = *reinterpret_cast<const floatx4*>(rr + vi * 4);
+            if (dr) {
+                if constexpr (sizeof(T) == 2) {
+                    const uint2 raw = *reinterpret_cast<const uint2*>(dr + vi * 4);
+                    r[0] += __builtin_bit_cast(float, raw.x << 16); r[1] += __builtin_bit_cast(float, raw.x & 0xffff0000u);
+                    r[2] += __builtin_bit_cast(float, raw.y << 16); r[3] += __builtin_bit_cast(float, raw.y & 0xffff0000u);
+                } else {
+                    const floatx4 dv = *reinterpret_cast<const floatx4*>(dr + vi * 4);
+                    r[0] += dv[0]; r[1] += dv[1]; r[2] += dv[2]; r[3] += dv[3];
+                }
+                *reinterpret_cast<floatx4*>(rr + vi * 4) = r;
+            }
+            v[it] = r;
+            ss += (r[0] * r[0] + r[1] * r[1]) + (r[2] * r[2] + r[3] * r[3]);
+        }
+    }
+    ss = warp_sum(ss);
+    if ((tid & 63) == 0) red[tid >> 6] = ss;
+    __syncthreads();
+    const float rinv = rsqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)d + eps);
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+        const int vi = it * 256 + tid;
+        if (vi < nvec) {
+            const floatx4 wv = *reinterpret_cast<const floatx4*>(w + vi * 4);
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = wv[e] * (v[it][e] * rinv);
+            if constexpr (sizeof(T) == 2) {
+                T e4[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) e4[e] = from_f32<T>(o[e]);
+                *reinterpret_cast<uint2*>(orow + vi * 4) = *reinterpret_cast<const uint2*>(e4);
+            } else {
+                *reinterpret_cast<floatx4*>(orow + vi * 4) = floatx4{o[0], o[1], o[2], o[3]};
+            }
+        }
+    }
 }
 
 int check_norm_common(const m2_rmsnorm_params* p, const char* what) {
@@ -370,7 +436,7 @@ extern "C" int m2_rmsnorm_gated_fwd(const m2_rmsnorm_params* p, void* stream) {
     a.x = p->x; a.x_sr = p->x_stride_row; a.z = p->z; a.z_sr = p->z_stride_row; a.w = p->weight;
     a.out = p->out; a.out_sr = p->out_stride_row; a.out_f32 = p->out_f32 || p->dtype == M2_F32;
     a.rows = p->rows; a.d = p->channels; a.gw = p->channels / p->n_groups; a.eps = p->eps;
-    a.rows_per_block = norm_rows_per_block(p->rows, p->n_groups, false);
+    a.rows_per_block = norm_rows_per_block_fwd(p->rows, p->n_groups, a.gw / V);
     hipStream_t st = static_cast<hipStream_t>(stream);
     M2_DISPATCH_DTYPE(p->dtype, T, return (launch_norm<T, false>(a, p->n_groups, st)));
     return M2_OK;
@@ -417,4 +483,26 @@ extern "C" int m2_rmsnorm_gated_bwd(const m2_rmsnorm_params* p, void* stream) {
     column_sum_kernel<<<(unsigned)ceil_div(p->channels, (int64_t)64), 1024, 0, st>>>(static_cast<const float*>(p->workspace), p->d_weight,
                                                                                      prows, p->channels);
     return check_launch("column_sum_kernel");
+}
+
+extern "C" int m2_add_rmsnorm(float* residual, int64_t residual_stride_row, const void* delta, int64_t delta_stride_row,
+                              const float* weight, void* out, int64_t out_stride_row, int64_t rows, int64_t channels, float eps,
+                              int32_t dtype, void* stream) {
+    using namespace m2;
+    M2_REQUIRE(rows >= 0 && channels > 0, M2_ERR_SHAPE, "add_rmsnorm: rows %lld, channels %lld", (long long)rows, (long long)channels);
+    M2_REQUIRE(channels % 4 == 0 && channels <= 8192, M2_ERR_SHAPE, "add_rmsnorm: channels %lld must be a multiple of 4, at most 8192",
+               (long long)channels);
+    M2_REQUIRE(dtype == M2_F32 || dtype == M2_BF16, M2_ERR_DTYPE, "add_rmsnorm: unsupported dtype %d", (int)dtype);
+    if (rows == 0) return M2_OK;
+    M2_REQUIRE(residual && weight && out, M2_ERR_NULL, "add_rmsnorm: residual, weight and out are required");
+    const size_t es = dtype == M2_F32 ? 4 : 2;
+    M2_REQUIRE(aligned16(residual) && aligned16(weight) && residual_stride_row % 4 == 0 && (uintptr_t)out % (4 * es) == 0 &&
+                   out_stride_row % 4 == 0 && (!delta || ((uintptr_t)delta % (4 * es) == 0 && delta_stride_row % 4 == 0)),
+               M2_ERR_ALIGN, "add_rmsnorm: rows must start on 4-element boundaries (residual and weight on 16 bytes)");
+    M2_REQUIRE(rows <= 0x7fffffff, M2_ERR_SHAPE, "add_rmsnorm: too many rows");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    M2_DISPATCH_DTYPE(dtype, T, (add_rmsnorm_kernel<T><<<(unsigned)rows, 256, 0, st>>>(residual, residual_stride_row, static_cast<const T*>(delta),
+                                                                                     delta_stride_row, weight, static_cast<T*>(out),
+                                                                                     out_stride_row, (int)channels, eps)));
+    return check_launch("add_rmsnorm_kernel");
 }

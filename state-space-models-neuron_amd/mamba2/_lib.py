@@ -4,6 +4,7 @@ The structures below mirror the C structs field for field.  ``load()`` raises if
 the library is missing: there is no CPU or PyTorch fallback in this package.
 """
 import ctypes as C
+import weakref
 import os
 
 import torch
@@ -89,6 +90,7 @@ SYMBOLS = {
     "m2_rmsnorm_gated_fwd": (C.c_int, [C.POINTER(RmsnormParams), _vp]),
     "m2_rmsnorm_gated_bwd_workspace_bytes": (_sz, [_i64, _i64, _i32, _i32]),
     "m2_rmsnorm_gated_bwd": (C.c_int, [C.POINTER(RmsnormParams), _vp]),
+    "m2_add_rmsnorm": (C.c_int, [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _i64, C.c_float, _i32, _vp]),
     "m2_mfma_selftest": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp]),
     "m2_stream_copy": (C.c_int, [_vp, _vp, _sz, _vp]),
 }
@@ -142,6 +144,27 @@ def require_gpu(*tensors):
     for t in tensors:
         if t is not None and not t.is_cuda:
             raise RuntimeError("mamba2 HIP kernels need tensors on a GPU device (got %s); there is no CPU path" % t.device)
+
+
+_f32_copies = {}          # id(tensor) -> (weak reference, key, fp32 copy); entries go when the tensor does
+
+
+def f32_param(t):
+    """fp32 contiguous values of a parameter-like tensor.  fp32 tensors are returned as they are.  For others (a model
+    held in bfloat16) the converted copy is kept while autograd is off (inference loops call the same kernels thousands
+    of times per second) and rebuilt when the tensor was written through autograd-visible in-place ops, moved or retyped;
+    writes through ``.data`` are not seen."""
+    if t.dtype == torch.float32:
+        return t.detach().contiguous()
+    if torch.is_grad_enabled():
+        return t.detach().float().contiguous()
+    key = (t.data_ptr(), t._version, t.dtype, tuple(t.shape))
+    ident = id(t)                     # the caller's tensor object (a module's Parameter lives as long as the module)
+    hit = _f32_copies.get(ident)
+    if hit is None or hit[0]() is not t or hit[1] != key:
+        hit = (weakref.ref(t, lambda _, i=ident: _f32_copies.pop(i, None)), key, t.detach().float().contiguous())
+        _f32_copies[ident] = hit
+    return hit[2]
 
 
 class Workspace:

@@ -144,7 +144,7 @@ def _norm_params(x, z, weight, n_groups, eps):
     p.rows, p.channels, p.n_groups = rows, d, n_groups
     p.dtype = _lib.dtype_code(x.dtype)
     p.eps = float(eps)
-    w32 = weight.detach().float().contiguous()
+    w32 = _lib.f32_param(weight)
     p.weight = _lib.ptr(w32)
     keep.append(w32)
     return p, keep
@@ -193,6 +193,35 @@ def rmsnorm_gated_bwd_hip(x, z, weight, d_out, n_groups, eps, out_dz=None):
         out_dz.copy_(dz)
         dz = out_dz
     return dx, dw, dz
+
+
+def add_rmsnorm_ok(channels, out_dtype):
+    """True if ``add_rmsnorm_`` takes rows of this width: a multiple of 4, at most 8192 channels, fp32 or bf16 output."""
+    return channels % 4 == 0 and 0 < channels <= 8192 and out_dtype in (torch.float32, torch.bfloat16)
+
+
+def add_rmsnorm_(residual, delta, weight, eps, out_dtype):
+    """``residual += delta`` in place (fp32), then RMSNorm of the sum, in one kernel (inference; the block boundary of the
+    token-by-token loop, ``modeling_mamba2.py:133-140`` + ``:94-103``).  ``delta`` (dtype ``out_dtype``) may be None.
+    Returns weight * residual * rsqrt(mean(residual^2) + eps) in ``out_dtype``."""
+    _lib.require_gpu(residual, delta, weight)
+    lib = _lib.load()
+    if residual.dtype != torch.float32 or not residual.is_contiguous():
+        raise ValueError("add_rmsnorm_: the residual stream must be contiguous float32")
+    rows, d, rsr = _rows2d(residual, "residual")
+    dsr = 0
+    if delta is not None:
+        if delta.shape != residual.shape or delta.dtype != out_dtype:
+            raise ValueError("add_rmsnorm_: delta must have the residual's shape and the output dtype")
+        if delta.stride(-1) != 1:
+            delta = delta.contiguous()
+        _, _, dsr = _rows2d(delta, "delta")
+    out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+    w32 = _lib.f32_param(weight)
+    rc = lib.m2_add_rmsnorm(_lib.ptr(residual), rsr, _lib.ptr(delta), dsr, _lib.ptr(w32), _lib.ptr(out), d, rows, d, float(eps),
+                            _lib.dtype_code(out_dtype), _lib.stream_ptr(residual.device))
+    _lib.check(rc, "m2_add_rmsnorm")
+    return out
 
 
 # --------------------------------------------------------------------------------------------- autograd form

@@ -171,9 +171,18 @@ class Mamba2Model(Mamba2PreTrainedModel):
         """input_ids: int64 (batch, 1), one token per sequence -> hidden states (batch, 1, hidden) after the final norm.
         The caller advances ``cache_params.seqlen_offset`` (a host integer, so that a captured step stays replayable)."""
         x = self.embeddings(input_ids)
+        act = self.layers[0].mixer.in_proj.weight.dtype if len(self.layers) else x.dtype
+        if not (self.config.residual_in_fp32 and not torch.is_grad_enabled() and x.is_cuda and glue.add_rmsnorm_ok(x.shape[-1], act)):
+            for mixer_block in self.layers:
+                x = mixer_block.step(x, cache_params=cache_params)
+            return self.norm_f(x)
+        # fp32 residual stream: each block's residual add and the next norm are one kernel (the same arithmetic as
+        # Mamba2Block.step followed by Mamba2RMSNorm: fp32 sum, fp32 norm, one rounding to the activation dtype)
+        residual, delta = x.float().contiguous(), None
         for mixer_block in self.layers:
-            x = mixer_block.step(x, cache_params=cache_params)
-        return self.norm_f(x)
+            normed = glue.add_rmsnorm_(residual, delta, mixer_block.norm.weight, mixer_block.norm.variance_epsilon, act)
+            delta = mixer_block.mixer.step(normed, cache_params=cache_params)
+        return glue.add_rmsnorm_(residual, delta, self.norm_f.weight, self.norm_f.variance_epsilon, act)
 
 
 class Mamba2ForCausalLM(Mamba2PreTrainedModel):

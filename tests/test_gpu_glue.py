@@ -120,6 +120,30 @@ def test_rmsnorm_gated_on_packed_views(dtype, width_pad):
     assert torch.equal(gpacked[..., d:], torch.full((b, l, extra), 3.0, dtype=dtype, device=DEV))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,d", [(128, 2560), (3, 4096), (1, 8192), (130, 100), (5, 1028)])
+def test_add_rmsnorm_in_place_residual(dtype, rows, d):
+    """residual += delta; out = w * residual * rsqrt(mean(residual^2) + eps): against the fp64 oracle norm of the fp64 sum."""
+    from mamba2 import glue
+    eps = 1e-5
+    res = _rand((rows, d), torch.float32, 31, scale=3.0)
+    delta = _rand((rows, d), dtype, 32)
+    w = 1.0 + 0.2 * _rand((d,), torch.float32, 33)
+    rg = res.to(DEV)
+    out = glue.add_rmsnorm_(rg, delta.to(DEV), w.to(DEV), eps, dtype)
+    s = res.double() + delta.double()
+    ref = rmsnorm_gated_ref(s, None, w.double(), 1, eps)
+    assert out.dtype == dtype and out.shape == (rows, d)
+    assert rel_rms_err(rg.cpu(), s) < 1e-6                     # the residual stream stays fp32
+    assert rel_rms_err(out.cpu(), ref) < TOL[dtype]
+    # nothing to add: the residual is left alone
+    before = rg.clone()
+    out2 = glue.add_rmsnorm_(rg, None, w.to(DEV), eps, dtype)
+    assert torch.equal(rg, before) and torch.equal(out2, out)
+    with pytest.raises(ValueError):
+        glue.add_rmsnorm_(torch.zeros(2, 8200, device=DEV), None, torch.ones(8200, device=DEV), eps, dtype)
+
+
 def test_glue_empty_and_errors():
     from mamba2 import glue
     x = torch.empty(0, 4, 512, dtype=torch.bfloat16, device=DEV)

@@ -113,6 +113,30 @@ def test_model_step_logits_equal_forward_logits(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("residual_in_fp32", [True, False])
+def test_model_step_equals_block_by_block_steps(dtype, residual_in_fp32):
+    """Mamba2Model.step (residual add fused with the next norm when the residual stream is fp32) against the blocks'
+    own step methods chained by hand (modeling_mamba2.py:337-350)."""
+    from mamba2.mamba2_mixer import Mamba2Cache
+    cfg, m = _model(dtype, layers=3, residual_in_fp32=residual_in_fp32)
+    b = 5
+    ids = torch.randint(0, cfg.vocab_size, (b, 6), generator=torch.Generator().manual_seed(7)).to(DEV)
+    c1 = Mamba2Cache(cfg, b, dtype=dtype, device=DEV)
+    c2 = Mamba2Cache(cfg, b, dtype=dtype, device=DEV)
+    with torch.no_grad():
+        for t in range(6):
+            got = m.backbone.step(ids[:, t:t + 1], c1)
+            x = m.backbone.embeddings(ids[:, t:t + 1])
+            for blk in m.backbone.layers:
+                x = blk.step(x, cache_params=c2)
+            ref = m.backbone.norm_f(x)
+            if dtype == torch.float32:
+                assert rel_err(got, ref) < 1e-5, t
+            else:
+                assert rel_rms_err(got, ref.float(), roundings=2) < 2e-2, t
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("W", [3, 4])
 @pytest.mark.parametrize("l1,l2", [(130, 40), (2, 131), (256, 1)])
 def test_prefill_hands_over_to_step_and_to_prefill(dtype, W, l1, l2):
