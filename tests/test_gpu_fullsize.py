@@ -4,7 +4,9 @@
   the second as initial state (forward), for the 2.7B (c1) and 7B-layer (c3) SSD shapes;
 * linearity of the backward in dy, and dD == sum(dy * x) (mamba2_kernel.py:471), at the c1 and c3 shapes;
 * conv: shifting the input by one token shifts the output by one token (causality + time invariance), c2 shape;
-* decode: 4 token steps from the prefill's final state == the chunked scan over the 4 extra tokens, c4 width.
+* decode: 4 token steps from the prefill's final state == the chunked scan over the 4 extra tokens, c4 width;
+* the whole mixer layer at the 7B-layer (c3) and 2.7B shapes: finite, batch rows independent;
+* two model layers at the 2.7B width: token-by-token path, prefill hand-off and captured step against the sequence forward.
 """
 import pytest
 import torch
@@ -99,3 +101,63 @@ def test_decode_continues_prefill_c4_width():
     assert rel_rms_err(y_dec, y_all[:, l:].float()) < 2e-2
     assert rel_rms_err(S, S_all) < 4e-2
     assert (S - S_all).norm() / S_all.norm() < 5e-3
+
+
+@pytest.mark.parametrize("hidden,heads,groups,b,l", [(4096, 128, 8, 2, 4096), (2560, 80, 1, 4, 2048)])
+def test_mixer_layer_full_shape_batch_rows_independent(hidden, heads, groups, b, l):
+    """The whole mixer layer (in_proj -> fused core -> out_proj) at the 7B-layer and 2.7B shapes, forward + backward:
+    finite, and every batch row computed alone gives what it gives inside the batch (outputs and input gradients; the
+    rows only meet in the parameter gradients)."""
+    from mamba2.configuration_mamba2 import Mamba2Config
+    from mamba2.mamba2_mixer import Mamba2Mixer
+    cfg = Mamba2Config(num_heads=heads, head_dim=64, hidden_size=hidden, state_size=128, n_groups=groups, num_hidden_layers=1)
+    torch.manual_seed(0)
+    with torch.device(DEV):
+        mix = Mamba2Mixer(cfg, 0).to(torch.bfloat16)
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    x = torch.randn(b, l, hidden, device=DEV, generator=gen).to(torch.bfloat16).requires_grad_(True)
+    dy = torch.randn(b, l, hidden, device=DEV, generator=gen).to(torch.bfloat16)
+    y = mix(x)
+    y.backward(dy)
+    assert torch.isfinite(y.float()).all() and torch.isfinite(x.grad.float()).all()
+    for name, p_ in mix.named_parameters():
+        assert p_.grad is not None and torch.isfinite(p_.grad.float()).all(), name
+    x1 = x.detach()[b - 1:].clone().requires_grad_(True)
+    y1 = mix(x1)
+    y1.backward(dy[b - 1:])
+    # the projections may pick different GEMM tiles for the one-row batch: the bf16 bar, not bit equality
+    assert rel_rms_err(y1, y.detach()[b - 1:].float(), roundings=2) < 2e-2
+    assert rel_rms_err(x1.grad, x.grad[b - 1:].float(), roundings=2) < 2e-2
+
+
+def test_model_step_full_width_two_layers():
+    """Two layers at the 2.7B width (d_model 2560, 80 heads, one group, n 128), bf16: the token-by-token path, the prefill
+    hand-off and the captured step against the sequence forward, on the kernels' fast paths for this head count."""
+    from mamba2.configuration_mamba2 import Mamba2Config
+    from mamba2.mamba2_mixer import Mamba2Cache
+    from mamba2.modeling_mamba2 import GraphedStep, Mamba2ForCausalLM
+    cfg = Mamba2Config(num_heads=80, head_dim=64, hidden_size=2560, state_size=128, n_groups=1, num_hidden_layers=2, vocab_size=1024,
+                       initializer_range=0.5)
+    torch.manual_seed(0)
+    with torch.device(DEV):
+        m = Mamba2ForCausalLM(cfg).to(torch.bfloat16).eval()
+    b, l1, l2 = 4, 200, 8
+    ids = torch.randint(0, cfg.vocab_size, (b, l1 + l2), device=DEV, generator=torch.Generator(device=DEV).manual_seed(2))
+
+    def close(got, ref):
+        g_, r_ = got.double(), ref.double()
+        return ((g_ - r_).norm() / r_.norm()).item() < 2e-2 and rel_rms_err(got.float(), ref.float()) < 0.2
+
+    with torch.no_grad():
+        full = m(input_ids=ids).logits
+        cache = Mamba2Cache(cfg, b, dtype=torch.bfloat16, device=DEV, conv_width=3)
+        pre = m(input_ids=ids[:, :l1], cache_params=cache, use_cache=True).logits
+        assert close(pre, full[:, :l1])
+        snap = [t.clone() for t in cache.conv_states + cache.ssm_states]
+        steps = torch.cat([m.step(ids[:, l1 + t:l1 + t + 1], cache) for t in range(l2)], dim=1)
+        assert close(steps, full[:, l1:])
+        for t, k in zip(cache.conv_states + cache.ssm_states, snap):
+            t.copy_(k)
+        graphed = GraphedStep(m, cache, b)
+        replayed = torch.cat([graphed(ids[:, l1 + t:l1 + t + 1]).clone() for t in range(l2)], dim=1)
+    assert torch.equal(replayed, steps)
