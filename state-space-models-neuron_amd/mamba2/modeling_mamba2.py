@@ -240,7 +240,9 @@ class GraphedStep:
     The graph reads the token ids from ``self.input_ids`` and the states from ``cache_params`` (updated in place by the
     decode kernel, so each replay continues from the last) and leaves the logits in ``self.logits``; ``__call__`` copies
     the ids in, replays and returns ``self.logits`` (overwritten by the next call).  The model's parameters and the cache
-    tensors must stay where they are while the object lives; ``cache_params`` may be reset or refilled by a prefill
+    tensors must stay where they are, and the parameters unchanged, while the object lives (the graph holds their
+    addresses, and for a model kept in bfloat16 the fp32 copies of the small per-head and norm parameters made before the
+    capture): build a new object after loading other weights.  ``cache_params`` may be reset or refilled by a prefill
     between replays.  The states advanced by the warm-up and capture runs are restored before ``__init__`` returns.
     """
 
