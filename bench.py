@@ -306,6 +306,49 @@ def cpu_baseline_ssd():
             "seconds_per_step": t}
 
 
+def _cpu_cores():
+    import torch
+    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+    torch.set_num_threads(cores)
+    return cores
+
+
+def cpu_baseline_conv():
+    """F.conv1d + SiLU with autograd (the conv oracle) on the host cores: the full conv workload, fp32."""
+    import torch
+    from oracle.conv import conv1d_grads_ref, make_conv_inputs
+    cores = _cpu_cores()
+    cfg = CONV_CFG
+    d = make_conv_inputs(cfg["b"], cfg["l"], cfg["C"], cfg["k"], seed=0, dtype=torch.float32)
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        conv1d_grads_ref(d["x"], d["w"], d["bias"], d["dy"], "silu")
+        times.append(time.perf_counter() - t0)
+    t = min(times[1:])
+    return {"value": cfg["b"] * cfg["l"] / t, "unit": "tokens/s", "cores": cores, "kind": "port", "seconds_per_step": t,
+            "sample": "full workload (b4 l2048 C5376 k4), fp32, F.conv1d + SiLU with autograd, 1 warm-up + best of 2"}
+
+
+def cpu_baseline_decode():
+    """The decode oracle on the host cores: 2 of the 64 layers at batch 128 (fp32), scaled by 32 to a whole step."""
+    import torch
+    from oracle.decode import decode_step_ref, make_decode_inputs
+    cores = _cpu_cores()
+    cfg = DEC_CFG
+    layers = 2
+    q = [make_decode_inputs(cfg["b"], cfg["h"], cfg["p"], cfg["n"], cfg["g"], cfg["k"], cfg["W"], seed=s) for s in range(layers)]
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for d in q:
+            decode_step_ref(d["xBC"], d["conv_state"], d["conv_weight"], d["conv_bias"], d["S"], d["dt"], d["A"], d["D"], n_groups=cfg["g"])
+        times.append(time.perf_counter() - t0)
+    t = min(times[1:]) * cfg["layers"] / layers
+    return {"value": t * 1e6, "unit": "us/step", "cores": cores, "kind": "port", "seconds_per_step": t,
+            "sample": "2 of the 64 layers (b128 h80 p64 n128, fp32, out-of-place oracle step), time scaled x32, 1 warm-up + best of 2"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -381,6 +424,15 @@ def main():
         out["other"] = other
     if not a.no_cpu and wanted("ssd"):
         out["cpu_baseline"] = cpu_baseline_ssd()
+    # the conv and decode oracles timed on the same host, next to their GPU lines
+    if not a.no_cpu:
+        for key, fn in (("conv1d", cpu_baseline_conv), ("decode", cpu_baseline_decode)):
+            tgt = out.get("other", {}).get(key) if key in out.get("other", {}) else (out if out.get("metric", "").startswith(key[:4]) else None)
+            if isinstance(tgt, dict) and "error" not in tgt:
+                try:
+                    tgt["cpu_baseline"] = fn()
+                except Exception as e:      # noqa: BLE001
+                    tgt["cpu_baseline"] = {"error": f"{type(e).__name__}: {e}"}
     print(json.dumps(out))
 
 
