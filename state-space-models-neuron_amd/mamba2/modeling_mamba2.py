@@ -234,6 +234,27 @@ class Mamba2ForCausalLM(Mamba2PreTrainedModel):
         return self.lm_head(hidden_states.to(self.lm_head.weight.dtype)).float()
 
 
+@torch.no_grad()
+def greedy_generate(model: "Mamba2ForCausalLM", input_ids, max_new_tokens: int, use_graph: bool = True, conv_width: Optional[int] = None):
+    """Greedy continuation of ``input_ids`` (batch, prompt_len) by ``max_new_tokens`` tokens: the prompt goes through the
+    sequence kernels once and leaves its states in a fresh cache (prefill), then every new token is one ``step`` --
+    replayed from one HIP graph when ``use_graph``.  The loop of ``mamba2_inference_no_tp.py:108-127`` with the prompt
+    prefilled instead of stepped through.  Returns (batch, prompt_len + max_new_tokens) token ids."""
+    b = input_ids.shape[0]
+    dtype = model.backbone.layers[0].mixer.in_proj.weight.dtype
+    cache = Mamba2Cache(model.config, b, dtype=dtype, device=input_ids.device, conv_width=conv_width)
+    logits = model(input_ids=input_ids, cache_params=cache, use_cache=True).logits[:, -1:]
+    step = GraphedStep(model, cache, b) if (use_graph and max_new_tokens > 1) else (lambda idx: model.step(idx, cache))
+    out = [input_ids]
+    for t in range(max_new_tokens):
+        nxt = logits.argmax(dim=-1)
+        out.append(nxt)
+        if t + 1 < max_new_tokens:
+            logits = step(nxt)
+            cache.seqlen_offset += 1
+    return torch.cat(out, dim=1)
+
+
 class GraphedStep:
     """``Mamba2ForCausalLM.step`` for one batch size, captured once into a HIP graph and replayed per token.
 

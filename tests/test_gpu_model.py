@@ -253,3 +253,20 @@ def test_decode_step_softplus_inside_matches_softplus_outside():
     y1, _, _ = mamba2_kernel_inference(q["xBC"], c1, q["conv_weight"], q["conv_bias"], S1, raw, q["A"], q["D"], n_groups=g, dt_bias=bias)
     y2, _, _ = mamba2_kernel_inference(q["xBC"], c2, q["conv_weight"], q["conv_bias"], S2, dt, q["A"], q["D"], n_groups=g)
     assert rel_err(y1, y2) < 1e-5 and rel_err(S1, S2) < 1e-5 and torch.equal(c1, c2)
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_greedy_generate_matches_recomputing_the_prefix(use_graph):
+    """Prefill + (captured) steps pick the same tokens as running the whole sequence again for every new token."""
+    from mamba2.modeling_mamba2 import greedy_generate
+    cfg, m = _model(torch.float32, layers=2)
+    prompt = torch.randint(0, cfg.vocab_size, (3, 37), generator=torch.Generator().manual_seed(8)).to(DEV)
+    got = greedy_generate(m, prompt, 12, use_graph=use_graph, conv_width=3)
+    seq = prompt
+    with torch.no_grad():
+        for _ in range(12):
+            logits = m(input_ids=seq).logits[:, -1]
+            top2 = logits.topk(2, dim=-1).values
+            assert ((top2[:, 0] - top2[:, 1]) > 1e-3).all(), "near tie: the comparison of token ids would not be meaningful"
+            seq = torch.cat([seq, logits.argmax(-1, keepdim=True)], dim=1)
+    assert got.shape == (3, 49) and torch.equal(got, seq)
