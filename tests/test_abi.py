@@ -117,3 +117,24 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libmamba2_hip.so")
     with pytest.raises(RuntimeError, match="no fallback"):
         _lib.load()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 2 and "one GPU only" in r.stderr and r.stdout.strip() == ""
+
+
+def test_f32_param_copy_is_kept_only_without_autograd():
+    from mamba2 import _lib
+    w = torch.nn.Parameter(torch.randn(8).bfloat16())
+    with torch.no_grad():
+        a, b = _lib.f32_param(w), _lib.f32_param(w)
+        assert a is b and torch.equal(a, w.float())
+        w.mul_(2)                                   # an in-place update (optimizer step, load_state_dict) is seen
+        c = _lib.f32_param(w)
+        assert c is not a and torch.equal(c, w.float())
+    assert _lib.f32_param(w) is not c               # autograd on: converted per call
+    f = torch.nn.Parameter(torch.randn(8))
+    assert _lib.f32_param(f).data_ptr() == f.data_ptr()
