@@ -192,9 +192,11 @@ class Mamba2ForCausalLM(Mamba2PreTrainedModel):
         super().__init__(config)
         self.backbone = Mamba2Model(config)
         self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
+        self.apply(self._init_weights)
+        # the head starts from the same normal law as the table (modeling_mamba2.py:366-377: init_method on the parallel linear)
+        nn.init.normal_(self.lm_head.weight, std=config.initializer_range)
         if config.tie_word_embeddings:
             self.lm_head.weight = self.backbone.embeddings.weight
-        self.apply(self._init_weights)
 
     def get_output_embeddings(self):
         return self.lm_head
