@@ -25,12 +25,14 @@ sys.path.insert(0, os.path.join(ROOT, "state-space-models-neuron_amd"))
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0     # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0              # MI355X HBM3E
-# Measured HBM bytes per step (rocprofv3 FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, the factors the 1 GiB copy kernel
-# gives in the same runs; profiles/bench_all_workloads_kernels.md).  They describe the kernels as profiled, not this run.
+# HBM bytes per step as PROFILED (two rocprofv3 --pmc runs of this file, FETCH_SIZE then WRITE_SIZE, each scaled by what
+# the same counter reads for the 1 GiB copy kernel in the same run; summaries under profiles/).  They are constants of
+# the kernels as last profiled, not measurements of this run: `traffic_source` in the JSON says so.
 SSD_TRAFFIC_BYTES = 1.441e9
 CONV_TRAFFIC_BYTES = 459.5e6
 DECODE_TRAFFIC_BYTES = 64 * 689.3e6
 GLUE_TRAFFIC_BYTES = 703.5e6
+TRAFFIC_SOURCE = "profiled constant: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this workload, scaled by the 1 GiB copy kernel; not measured in this run"
 
 SSD_CFG = dict(b=4, l=2048, h=80, p=64, n=128, g=1)
 CONV_CFG = dict(b=4, l=2048, C=5376, k=4)
@@ -41,6 +43,25 @@ Q = 128
 def ssd_flops_fwd(b, l, h, p, n, g):
     c = math.ceil(l / Q)
     return b * c * (h * (2 * Q * Q * p + 4 * Q * n * p) + g * 2 * Q * Q * n)
+
+
+def parity_entry(got, ref):
+    """Raw acceptance figures of one tensor against the oracle: max|err| / RMS(ref) (the bf16 bar is 2e-2, plus, for a
+    tensor stored in bf16, `bf16_floor` = what storing the exact value costs) and the relative L2 error."""
+    import torch
+    ref = ref.double().cpu()
+    got_d = got.detach().double().cpu()
+    rms = ref.pow(2).mean().sqrt().clamp_min(1e-30)
+    raw = ((got_d - ref).abs().max() / rms).item()
+    floor = ((ref.to(torch.bfloat16).double() - ref).abs().max() / rms).item() if got.dtype == torch.bfloat16 else 0.0
+    l2 = ((got_d - ref).norm() / ref.norm().clamp_min(1e-30)).item()
+    return {"raw": round(raw, 5), "bf16_floor": round(floor, 5), "rel_l2": round(l2, 6), "ok": bool(raw < 2e-2 + floor and l2 < 1e-2)}
+
+
+def require_parity(name, table):
+    bad = {k: v for k, v in table.items() if not v["ok"]}
+    if bad:
+        raise RuntimeError(f"{name}: outputs differ from the oracle, nothing timed: {bad}")
 
 
 def event_time_ms(fn, steps, warmup):
@@ -61,11 +82,35 @@ def event_time_ms(fn, steps, warmup):
     return wall, per
 
 
-def bench_ssd(steps, warmup):
+def check_ssd(cfg, ref=None):
+    """The HIP forward + backward against the oracle on the same seeded bf16 inputs, before anything is timed.  `ref`:
+    oracle results already computed for cfg by the CPU-baseline leg (fp32 arithmetic on the same inputs)."""
+    import torch
+    from mamba2.mamba2_kernel import alloc_chunk_states, ssd_backward, ssd_forward
+    from oracle.ssd import make_ssd_inputs, ssd_grads_ref
+    d = make_ssd_inputs(cfg["b"], cfg["l"], cfg["h"], cfg["p"], cfg["n"], cfg["g"], seed=0, dtype=torch.bfloat16)
+    if ref is None:
+        ref = ssd_grads_ref(*(d[k].double() for k in ("dt", "A", "X", "B", "C", "D", "dy")), chunk=Q)
+    g = {k: v.to("cuda:0") for k, v in d.items()}
+    st = alloc_chunk_states(g["dt"], g["A"], g["X"], g["B"], g["C"])
+    y, S = ssd_forward(g["dt"], g["A"], g["X"], g["B"], g["C"], g["D"], want_final_state=True, chunk_states=st)
+    ddt, dA, dX, dB, dC, dD, _ = ssd_backward(g["dt"], g["A"], g["X"], g["B"], g["C"], g["D"], g["dy"], chunk_states=st)
+    got = {"y": y, "dX": dX, "ddt": ddt, "dB": dB, "dC": dC, "dA": dA, "dD": dD}
+    table = {k: parity_entry(v, ref[k]) for k, v in got.items()}
+    # the final state is an fp32 sum of MFMA products with bf16-rounded operands: reported, held to the relative-L2 bound
+    fs = parity_entry(S, ref["final_state"])
+    fs["ok"] = bool(fs["rel_l2"] < 1e-2)
+    table["final_state"] = fs
+    require_parity("ssd", table)
+    return table
+
+
+def bench_ssd(steps, warmup, ref=None, check_cfg=None):
     import torch
     from mamba2.mamba2_kernel import SAVE_CHUNK_STATES, alloc_chunk_states, ssd_backward, ssd_forward
     from oracle.ssd import make_ssd_inputs
     cfg = SSD_CFG
+    parity = check_ssd(check_cfg or cfg, ref)
     d = make_ssd_inputs(cfg["b"], cfg["l"], cfg["h"], cfg["p"], cfg["n"], cfg["g"], seed=0, dtype=torch.bfloat16, device="cuda:0")
     # what Mamba2Kernel.forward/backward do: the forward keeps the chunk states and operand tiles for the backward (102 MB here)
     states = alloc_chunk_states(d["dt"], d["A"], d["X"], d["B"], d["C"]) if SAVE_CHUNK_STATES else None
@@ -81,7 +126,8 @@ def bench_ssd(steps, warmup):
     flops = 3 * ssd_flops_fwd(**cfg)
     io_bytes = 2 * (5 * cfg["b"] * cfg["l"] * cfg["h"] * cfg["p"] + 4 * cfg["b"] * cfg["l"] * cfg["g"] * cfg["n"] + 2 * cfg["b"] * cfg["l"] * cfg["h"])
     return dict(ms_per_step=wall_ms, ms_event_avg=ms, ms_event_min=per[0], ms_event_median=per[len(per) // 2],
-                tokens_per_s=tokens / (wall_ms * 1e-3), flops=flops, io_bytes=io_bytes, tflops=flops / (ms * 1e-3) / 1e12, tokens=tokens)
+                tokens_per_s=tokens / (wall_ms * 1e-3), flops=flops, io_bytes=io_bytes, tflops=flops / (ms * 1e-3) / 1e12, tokens=tokens,
+                parity=parity, parity_shape="b{b} l{l} h{h} p{p} n{n} g{g}".format(**(check_cfg or cfg)))
 
 
 def bench_conv(steps, warmup):
@@ -93,6 +139,15 @@ def bench_conv(steps, warmup):
     sets = [make_conv_inputs(cfg["b"], cfg["l"], cfg["C"], cfg["k"], seed=s, dtype=torch.bfloat16, device="cuda:0") for s in range(nsets)]
     outs = [torch.empty_like(sets[0]["x"]) for _ in range(2)]
     state = {"i": 0}
+    # the full workload against the oracle (F.conv1d + SiLU + autograd, fp64) before timing
+    from oracle.conv import conv1d_grads_ref
+    c0 = {k: v.cpu().double() for k, v in sets[0].items()}
+    y_ref, dx_ref, dw_ref, db_ref = conv1d_grads_ref(c0["x"], c0["w"], c0["bias"], c0["dy"], "silu")
+    y0 = conv1d_forward(sets[0]["x"], sets[0]["w"], sets[0]["bias"], "silu", channels_last=True)
+    dx0, dw0, db0 = conv1d_backward(sets[0]["x"], sets[0]["w"], sets[0]["bias"], sets[0]["dy"], "silu", channels_last=True)
+    parity = {"y": parity_entry(y0, y_ref), "dx": parity_entry(dx0, dx_ref), "dw": parity_entry(dw0, dw_ref), "db": parity_entry(db0, db_ref)}
+    require_parity("conv1d", parity)
+    del c0, y_ref, dx_ref, y0, dx0
 
     def step():
         d = sets[state["i"] % nsets]
@@ -106,9 +161,9 @@ def bench_conv(steps, warmup):
     bytes_ = elems * 2 * 5          # fwd: read x, write y; bwd: read x, dy, write dx
     tokens = cfg["b"] * cfg["l"]
     return dict(metric="conv1d+SiLU fwd+bwd tokens/s", value=tokens / (ms * 1e-3), unit="tokens/s", ms_per_step=ms, dtype="bf16",
-                config={"workload": "depthwise conv1d k=4 + SiLU fwd+bwd, b4 l2048 C5376, channels-last"},
+                config={"workload": "depthwise conv1d k=4 + SiLU fwd+bwd, b4 l2048 C5376, channels-last"}, parity=parity,
                 roofline={"bound": "hbm", "achieved": bytes_ / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": CONV_TRAFFIC_BYTES,
+                          "frac": bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": CONV_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
                           "algorithmic_bytes_per_step": bytes_, "kernels": "conv_fwd_cl_kernel + conv_bwd_cl_kernel + conv_reduce_partials_kernel"})
 
 
@@ -149,7 +204,7 @@ def bench_glue(steps, warmup):
                 dtype="bf16 I/O, f32 arithmetic",
                 config={"workload": "gated RMSNorm d5120 g1 + softplus(dt + bias) h80, fwd+bwd, b4 l2048, packed-buffer column slices"},
                 roofline={"bound": "hbm", "achieved": bytes_ / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": GLUE_TRAFFIC_BYTES,
+                          "frac": bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": GLUE_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
                           "algorithmic_bytes_per_step": bytes_,
                           "kernels": "rmsnorm_gated_kernel fwd + bwd, column_sum_kernel, softplus_fwd_kernel, softplus_bwd_kernel"})
 
@@ -201,6 +256,17 @@ def bench_decode(steps, warmup):
     # distinct state buffers per layer (21.5 GB of fp32 SSM state): nothing is served from cache
     S = [0.1 * torch.randn(cfg["b"], cfg["h"], cfg["p"], cfg["n"], device="cuda:0", generator=gen) for _ in range(L)]
     conv = [torch.randn(cfg["b"], d["xBC"].shape[-1], cfg["W"], device="cuda:0", generator=gen).to(torch.bfloat16) for _ in range(L)]
+    # one layer against the oracle (fp64 on the host) before timing: y, the updated SSM state and the shifted conv state
+    from oracle.decode import decode_step_ref
+    S0, c0 = S[0].clone(), conv[0].clone()
+    y_ref, cs_ref, S_ref = decode_step_ref(*(t.cpu().double() for t in (d["xBC"], c0, d["conv_weight"], d["conv_bias"], S0, d["dt"], d["A"], d["D"])),
+                                           n_groups=cfg["g"])
+    y0, c1, S1 = mamba2_kernel_inference(d["xBC"], c0, d["conv_weight"], d["conv_bias"], S0, d["dt"], d["A"], d["D"], n_groups=cfg["g"])
+    parity = {"y": parity_entry(y0, y_ref), "S": parity_entry(S1, S_ref)}
+    parity["S"]["ok"] = bool(parity["S"]["raw"] < 1e-4)
+    parity["conv_state_bit_exact"] = {"ok": bool(torch.equal(c1.cpu().double(), cs_ref))}
+    require_parity("decode", parity)
+    del S0, c0, y_ref, cs_ref, S_ref, S1
 
     def step():
         for i in range(L):
@@ -213,9 +279,9 @@ def bench_decode(steps, warmup):
     bytes_ = per_layer * L
     return dict(metric="decode token-step latency (64 layers, batch 128)", value=ms * 1e3, unit="us/step", higher_is_better=False,
                 us_per_sequence_token=ms * 1e3 / cfg["b"], ms_per_step=ms, wall_ms_per_step=wall_ms, dtype="f32 state / bf16 activations",
-                config={"workload": "decode step, 64 layers x (b128, h80, p64, n128, C5376, W3), states in place"},
+                config={"workload": "decode step, 64 layers x (b128, h80, p64, n128, C5376, W3), states in place"}, parity=parity,
                 roofline={"bound": "hbm", "achieved": bytes_ / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": DECODE_TRAFFIC_BYTES,
+                          "frac": bytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": DECODE_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
                           "algorithmic_bytes_per_step": bytes_, "kernels": "decode_conv_kernel + decode_ssm_kernel, 64 launches each"})
 
 
@@ -287,30 +353,49 @@ def bench_copy(steps, warmup):
                           "kernels": "stream_copy_kernel"})
 
 
-def cpu_baseline_ssd():
-    """The pure-PyTorch chunked oracle (fp32, autograd) on the host cores: the full headline configuration."""
-    import torch
-    from oracle.ssd import make_ssd_inputs, ssd_grads_ref
-    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
-    torch.set_num_threads(cores)
-    cfg = SSD_CFG
-    d = make_ssd_inputs(cfg["b"], cfg["l"], cfg["h"], cfg["p"], cfg["n"], cfg["g"], seed=0, dtype=torch.float32)
-    times = []
-    for i in range(3):
-        t0 = time.perf_counter()
-        ssd_grads_ref(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], d["dy"], chunk=Q)
-        times.append(time.perf_counter() - t0)
-    t = sorted(times[1:])[0] if len(times) > 1 else times[0]
-    return {"value": cfg["b"] * cfg["l"] / t, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": "full workload (b4 l2048 h80 p64 n128), fp32, chunked-matmul oracle with autograd, 1 warm-up + best of 2",
-            "seconds_per_step": t}
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def _cpu_cores():
+    """Threads the CPU legs use: the box's CPU share (OMP_NUM_THREADS there), else every core the host reports."""
     import torch
-    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
     torch.set_num_threads(cores)
     return cores
+
+
+def _cpu_info(cores):
+    return {"cores": cores, "host_cpu_count": os.cpu_count(), "cpu_model": cpu_model()}
+
+
+def cpu_baseline_ssd():
+    """The pure-PyTorch chunked oracle (fp32 arithmetic, autograd) on the host cores: the full headline configuration,
+    on the same seeded bf16-rounded inputs the GPU path gets.  Returns (baseline record, the oracle's results)."""
+    import torch
+    from oracle.ssd import make_ssd_inputs, ssd_grads_ref
+    cores = _cpu_cores()
+    cfg = SSD_CFG
+    d = make_ssd_inputs(cfg["b"], cfg["l"], cfg["h"], cfg["p"], cfg["n"], cfg["g"], seed=0, dtype=torch.bfloat16)
+    d = {k: v.float() for k, v in d.items()}
+    times = []
+    for i in range(3):
+        t0 = time.perf_counter()
+        ref = ssd_grads_ref(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"], d["dy"], chunk=Q)
+        times.append(time.perf_counter() - t0)
+    t = sorted(times[1:])[0] if len(times) > 1 else times[0]
+    rec = {"value": cfg["b"] * cfg["l"] / t, "unit": "tokens/s", "kind": "port",
+           "sample": "full workload (b4 l2048 h80 p64 n128), fp32, chunked-matmul oracle with autograd, 1 warm-up + best of 2",
+           "seconds_per_step": t}
+    rec.update(_cpu_info(cores))
+    return rec, ref
 
 
 def cpu_baseline_conv():
@@ -326,8 +411,10 @@ def cpu_baseline_conv():
         conv1d_grads_ref(d["x"], d["w"], d["bias"], d["dy"], "silu")
         times.append(time.perf_counter() - t0)
     t = min(times[1:])
-    return {"value": cfg["b"] * cfg["l"] / t, "unit": "tokens/s", "cores": cores, "kind": "port", "seconds_per_step": t,
-            "sample": "full workload (b4 l2048 C5376 k4), fp32, F.conv1d + SiLU with autograd, 1 warm-up + best of 2"}
+    rec = {"value": cfg["b"] * cfg["l"] / t, "unit": "tokens/s", "kind": "port", "seconds_per_step": t,
+           "sample": "full workload (b4 l2048 C5376 k4), fp32, F.conv1d + SiLU with autograd, 1 warm-up + best of 2"}
+    rec.update(_cpu_info(cores))
+    return rec
 
 
 def cpu_baseline_decode():
@@ -345,8 +432,10 @@ def cpu_baseline_decode():
             decode_step_ref(d["xBC"], d["conv_state"], d["conv_weight"], d["conv_bias"], d["S"], d["dt"], d["A"], d["D"], n_groups=cfg["g"])
         times.append(time.perf_counter() - t0)
     t = min(times[1:]) * cfg["layers"] / layers
-    return {"value": t * 1e6, "unit": "us/step", "cores": cores, "kind": "port", "seconds_per_step": t,
-            "sample": "2 of the 64 layers (b128 h80 p64 n128, fp32, out-of-place oracle step), time scaled x32, 1 warm-up + best of 2"}
+    rec = {"value": t * 1e6, "unit": "us/step", "kind": "port", "seconds_per_step": t,
+           "sample": "2 of the 64 layers (b128 h80 p64 n128, fp32, out-of-place oracle step), time scaled x32, 1 warm-up + best of 2"}
+    rec.update(_cpu_info(cores))
+    return rec
 
 
 def main():
@@ -377,14 +466,22 @@ def main():
         return a.workload == name or (a.workload == "all" and name not in skip)
 
     if wanted("ssd"):
-        r = bench_ssd(a.steps, a.warmup)
+        # the CPU leg runs first: its results (the oracle on the same inputs) are what the HIP outputs are checked against
+        # before anything is timed; without it the check runs on a quarter of the batch and sequence
+        cpu_rec, ref, check_cfg = None, None, None
+        if a.no_cpu:
+            check_cfg = dict(SSD_CFG, b=1, l=512)
+        else:
+            cpu_rec, ref = cpu_baseline_ssd()
+        r = bench_ssd(a.steps, a.warmup, ref, check_cfg)
+        del ref
         out.update({
             "metric": "SSD fwd+bwd tokens/s", "value": r["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1,
             "steps": a.steps, "warmup": a.warmup, "ms_per_step": r["ms_per_step"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "Mamba-2 2.7B-shaped SSD chunked scan fwd+bwd: b4 l2048 h80 p64 n128 g1 chunk128, bf16 I/O, fp32 state"},
             "roofline": {"bound": "mfma", "achieved": r["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": r["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": SSD_TRAFFIC_BYTES,
+                         "frac": r["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": SSD_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
                          "algorithmic_flops_per_step": r["flops"], "event_ms_avg": r["ms_event_avg"],
                          "event_ms_min": r["ms_event_min"],
                          "kernels": "all launches of m2_ssd_fwd + m2_ssd_bwd (one step), HIP events on the launch stream"},
@@ -392,7 +489,11 @@ def main():
             "roofline_hbm": {"bound": "hbm", "achieved": r["io_bytes"] / (r["ms_event_avg"] * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                              "frac": r["io_bytes"] / (r["ms_event_avg"] * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": SSD_TRAFFIC_BYTES,
                              "traffic_rate": SSD_TRAFFIC_BYTES / (r["ms_event_avg"] * 1e-3) / 1e9, "algorithmic_bytes_per_step": r["io_bytes"]},
+            "parity": {"against": "oracle.ssd.ssd_grads_ref on the same seeded inputs, " + r["parity_shape"] + ", checked before timing",
+                       "tensors": r["parity"]},
         })
+        if cpu_rec is not None:
+            out["cpu_baseline"] = cpu_rec
     def secondary(key, fn, *args):
         # with --workload all a failure in a secondary workload is reported in its place and does not take the headline
         # line with it; asked for by name, it fails loudly
@@ -422,8 +523,6 @@ def main():
         out.setdefault("higher_is_better", True)
     if other:
         out["other"] = other
-    if not a.no_cpu and wanted("ssd"):
-        out["cpu_baseline"] = cpu_baseline_ssd()
     # the conv and decode oracles timed on the same host, next to their GPU lines
     if not a.no_cpu:
         for key, fn in (("conv1d", cpu_baseline_conv), ("decode", cpu_baseline_decode)):

@@ -59,6 +59,10 @@ extern "C" {
 /* ABI version of this header; bumped on any incompatible change. */
 int m2_abi_version(void);
 const char* m2_last_error(void);
+/* Layout of a parameter structure as THIS library was compiled: out[0] = sizeof, out[1..] = offsetof each field in
+ * declaration order.  which: 0 m2_conv1d_params, 1 m2_ssd_params, 2 m2_decode_params, 3 m2_rmsnorm_params.  Returns the
+ * number of entries (only the first `capacity` are written); a binding compares them with its own mirror of the structs. */
+int m2_struct_layout(int32_t which, int64_t* out, int32_t capacity);
 
 /* ------------------------------------------------------------------ conv1d
  * y[b,t,c] = act(bias[c] + sum_{i<k} w[c,i] * x[b,t-(k-1)+i,c]),  x[t<0] = 0.
@@ -174,7 +178,7 @@ int m2_decode_step(const m2_decode_params* p, void* stream);
  * rmsnorm:   h = x * silu(z) (h = x without z);  out = weight * h * rsqrt(mean(h^2) + eps) with the mean
  *            taken inside each of n_groups groups of channels / n_groups contiguous channels.
  *            Backward: dx, dz (same type as x) and d_weight (fp32, summed over the rows).
- *            Channels per group: a multiple of 8 (bf16) / 4 (fp32), at most 8192 (bf16) / 4096 (fp32).
+ *            Channels per group: a multiple of 8 (bf16) / 4 (fp32), at most 8192.
  * dt_bias, weight, d_bias, d_weight are fp32.  The backward entry points take a workspace of
  * m2_*_bwd_workspace_bytes() bytes (per-block partial sums, added in a fixed order: no atomics).
  */

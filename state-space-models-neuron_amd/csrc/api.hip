@@ -60,15 +60,92 @@ mfma_selftest_kernel(const T* __restrict__ A, const T* __restrict__ Bt, float* _
             }
 }
 
-__global__ void __launch_bounds__(256) stream_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n) {
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+// A workgroup copies blocks of 256 x 4 vectors: four 16-byte loads in flight per lane, each a whole 4 KiB run per wave
+// pair, streamed past the caches on both sides (nothing is read twice).
+__global__ void __launch_bounds__(256) stream_copy_kernel(const floatx4* __restrict__ src, floatx4* __restrict__ dst, size_t n) {
+    constexpr size_t kBlock = 256 * 4;
+    const size_t nblk = n / kBlock;
+    for (size_t b = blockIdx.x; b < nblk; b += gridDim.x) {
+        const floatx4* s = src + b * kBlock + threadIdx.x;
+        floatx4* d = dst + b * kBlock + threadIdx.x;
+        floatx4 v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = __builtin_nontemporal_load(s + q * 256);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) __builtin_nontemporal_store(v[q], d + q * 256);
+    }
+    if (blockIdx.x == 0)
+        for (size_t i = nblk * kBlock + threadIdx.x; i < n; i += 256) dst[i] = src[i];
 }
+
+#define M2_OFF(s, f) (int64_t)offsetof(s, f)
+static const int64_t k_layout_0[] = {(int64_t)sizeof(m2_conv1d_params),
+    M2_OFF(m2_conv1d_params, x), M2_OFF(m2_conv1d_params, w), M2_OFF(m2_conv1d_params, bias), M2_OFF(m2_conv1d_params, dy),
+    M2_OFF(m2_conv1d_params, y), M2_OFF(m2_conv1d_params, dx), M2_OFF(m2_conv1d_params, dw), M2_OFF(m2_conv1d_params, db),
+    M2_OFF(m2_conv1d_params, workspace), M2_OFF(m2_conv1d_params, workspace_bytes), M2_OFF(m2_conv1d_params, batch),
+    M2_OFF(m2_conv1d_params, seqlen), M2_OFF(m2_conv1d_params, channels), M2_OFF(m2_conv1d_params, k),
+    M2_OFF(m2_conv1d_params, x_stride_b), M2_OFF(m2_conv1d_params, x_stride_l), M2_OFF(m2_conv1d_params, x_stride_c),
+    M2_OFF(m2_conv1d_params, y_stride_b), M2_OFF(m2_conv1d_params, y_stride_l), M2_OFF(m2_conv1d_params, y_stride_c),
+    M2_OFF(m2_conv1d_params, dx_stride_b), M2_OFF(m2_conv1d_params, dx_stride_l), M2_OFF(m2_conv1d_params, dx_stride_c),
+    M2_OFF(m2_conv1d_params, dtype), M2_OFF(m2_conv1d_params, param_dtype), M2_OFF(m2_conv1d_params, activation),};
+static const int64_t k_layout_1[] = {(int64_t)sizeof(m2_ssd_params),
+    M2_OFF(m2_ssd_params, x), M2_OFF(m2_ssd_params, dt), M2_OFF(m2_ssd_params, A), M2_OFF(m2_ssd_params, B),
+    M2_OFF(m2_ssd_params, C), M2_OFF(m2_ssd_params, D), M2_OFF(m2_ssd_params, initial_state), M2_OFF(m2_ssd_params, final_state),
+    M2_OFF(m2_ssd_params, chunk_states), M2_OFF(m2_ssd_params, y), M2_OFF(m2_ssd_params, dy),
+    M2_OFF(m2_ssd_params, d_final_state), M2_OFF(m2_ssd_params, dx), M2_OFF(m2_ssd_params, ddt), M2_OFF(m2_ssd_params, dA),
+    M2_OFF(m2_ssd_params, dB), M2_OFF(m2_ssd_params, dC), M2_OFF(m2_ssd_params, dD), M2_OFF(m2_ssd_params, d_initial_state),
+    M2_OFF(m2_ssd_params, workspace), M2_OFF(m2_ssd_params, workspace_bytes), M2_OFF(m2_ssd_params, batch),
+    M2_OFF(m2_ssd_params, seqlen), M2_OFF(m2_ssd_params, nheads), M2_OFF(m2_ssd_params, headdim), M2_OFF(m2_ssd_params, dstate),
+    M2_OFF(m2_ssd_params, ngroups), M2_OFF(m2_ssd_params, x_stride_b), M2_OFF(m2_ssd_params, x_stride_l),
+    M2_OFF(m2_ssd_params, x_stride_h), M2_OFF(m2_ssd_params, dt_stride_b), M2_OFF(m2_ssd_params, dt_stride_l),
+    M2_OFF(m2_ssd_params, B_stride_b), M2_OFF(m2_ssd_params, B_stride_l), M2_OFF(m2_ssd_params, B_stride_g),
+    M2_OFF(m2_ssd_params, C_stride_b), M2_OFF(m2_ssd_params, C_stride_l), M2_OFF(m2_ssd_params, C_stride_g),
+    M2_OFF(m2_ssd_params, y_stride_b), M2_OFF(m2_ssd_params, y_stride_l), M2_OFF(m2_ssd_params, y_stride_h),
+    M2_OFF(m2_ssd_params, dy_stride_b), M2_OFF(m2_ssd_params, dy_stride_l), M2_OFF(m2_ssd_params, dy_stride_h),
+    M2_OFF(m2_ssd_params, dx_stride_b), M2_OFF(m2_ssd_params, dx_stride_l), M2_OFF(m2_ssd_params, dx_stride_h),
+    M2_OFF(m2_ssd_params, ddt_stride_b), M2_OFF(m2_ssd_params, ddt_stride_l), M2_OFF(m2_ssd_params, dB_stride_b),
+    M2_OFF(m2_ssd_params, dB_stride_l), M2_OFF(m2_ssd_params, dB_stride_g), M2_OFF(m2_ssd_params, dC_stride_b),
+    M2_OFF(m2_ssd_params, dC_stride_l), M2_OFF(m2_ssd_params, dC_stride_g), M2_OFF(m2_ssd_params, dtype),
+    M2_OFF(m2_ssd_params, dt_dtype), M2_OFF(m2_ssd_params, dt_bias), M2_OFF(m2_ssd_params, d_dt_bias),};
+static const int64_t k_layout_2[] = {(int64_t)sizeof(m2_decode_params),
+    M2_OFF(m2_decode_params, xBC), M2_OFF(m2_decode_params, conv_state), M2_OFF(m2_decode_params, conv_w),
+    M2_OFF(m2_decode_params, conv_b), M2_OFF(m2_decode_params, S), M2_OFF(m2_decode_params, dt), M2_OFF(m2_decode_params, A),
+    M2_OFF(m2_decode_params, D), M2_OFF(m2_decode_params, y), M2_OFF(m2_decode_params, workspace),
+    M2_OFF(m2_decode_params, workspace_bytes), M2_OFF(m2_decode_params, batch), M2_OFF(m2_decode_params, nheads),
+    M2_OFF(m2_decode_params, headdim), M2_OFF(m2_decode_params, dstate), M2_OFF(m2_decode_params, ngroups),
+    M2_OFF(m2_decode_params, k), M2_OFF(m2_decode_params, W), M2_OFF(m2_decode_params, xBC_stride_b),
+    M2_OFF(m2_decode_params, dt_stride_b), M2_OFF(m2_decode_params, y_stride_b), M2_OFF(m2_decode_params, dtype),
+    M2_OFF(m2_decode_params, param_dtype), M2_OFF(m2_decode_params, activation), M2_OFF(m2_decode_params, dt_bias),};
+static const int64_t k_layout_3[] = {(int64_t)sizeof(m2_rmsnorm_params),
+    M2_OFF(m2_rmsnorm_params, x), M2_OFF(m2_rmsnorm_params, z), M2_OFF(m2_rmsnorm_params, weight),
+    M2_OFF(m2_rmsnorm_params, out), M2_OFF(m2_rmsnorm_params, d_out), M2_OFF(m2_rmsnorm_params, dx),
+    M2_OFF(m2_rmsnorm_params, dz), M2_OFF(m2_rmsnorm_params, d_weight), M2_OFF(m2_rmsnorm_params, workspace),
+    M2_OFF(m2_rmsnorm_params, workspace_bytes), M2_OFF(m2_rmsnorm_params, rows), M2_OFF(m2_rmsnorm_params, channels),
+    M2_OFF(m2_rmsnorm_params, x_stride_row), M2_OFF(m2_rmsnorm_params, z_stride_row), M2_OFF(m2_rmsnorm_params, out_stride_row),
+    M2_OFF(m2_rmsnorm_params, d_out_stride_row), M2_OFF(m2_rmsnorm_params, dx_stride_row),
+    M2_OFF(m2_rmsnorm_params, dz_stride_row), M2_OFF(m2_rmsnorm_params, n_groups), M2_OFF(m2_rmsnorm_params, dtype),
+    M2_OFF(m2_rmsnorm_params, out_f32), M2_OFF(m2_rmsnorm_params, eps),};
+#undef M2_OFF
 
 }  // namespace
 }  // namespace m2
 
-extern "C" int m2_abi_version(void) { return 3; }
+extern "C" int m2_abi_version(void) { return 4; }
+
+extern "C" int m2_struct_layout(int32_t which, int64_t* out, int32_t capacity) {
+    using namespace m2;
+    const int64_t* tab = nullptr;
+    int n = 0;
+    switch (which) {
+        case 0: tab = k_layout_0; n = (int)(sizeof(k_layout_0) / sizeof(int64_t)); break;
+        case 1: tab = k_layout_1; n = (int)(sizeof(k_layout_1) / sizeof(int64_t)); break;
+        case 2: tab = k_layout_2; n = (int)(sizeof(k_layout_2) / sizeof(int64_t)); break;
+        case 3: tab = k_layout_3; n = (int)(sizeof(k_layout_3) / sizeof(int64_t)); break;
+        default: return fail(M2_ERR_SHAPE, "struct_layout: unknown structure %d", (int)which);
+    }
+    for (int i = 0; i < n && i < capacity; ++i) out[i] = tab[i];
+    return n;
+}
 extern "C" const char* m2_last_error(void) { return m2::g_err; }
 
 extern "C" int m2_mfma_selftest(const void* A, const void* Bt, float* C, int64_t M, int64_t N, int64_t K, int32_t dtype, void* stream) {
@@ -91,8 +168,8 @@ extern "C" int m2_stream_copy(const void* src, void* dst, size_t bytes, void* st
     M2_REQUIRE(bytes % 16 == 0 && aligned16(src) && aligned16(dst), M2_ERR_ALIGN, "stream_copy: size and pointers must be multiples of 16 bytes");
     if (bytes == 0) return M2_OK;
     const size_t n = bytes / 16;
-    size_t blocks = (n + 255) / 256;
-    if (blocks > 256 * 16) blocks = 256 * 16;
-    stream_copy_kernel<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const uint4*>(src), static_cast<uint4*>(dst), n);
+    size_t blocks = (n + 1023) / 1024;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    stream_copy_kernel<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const floatx4*>(src), static_cast<floatx4*>(dst), n);
     return check_launch("stream_copy");
 }

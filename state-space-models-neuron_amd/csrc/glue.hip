@@ -285,10 +285,11 @@ int64_t norm_rows_per_block_fwd(int64_t rows, int64_t groups, int64_t nvec) {
     return norm_rows_per_block(rows, groups, false);
 }
 // waves per (row, group) and vectors per lane for a group of `nvec` 16-byte vectors; false if it does not fit
-bool norm_shape(int64_t nvec, int* wpg, int* nv) {
+bool norm_shape(int64_t nvec, int vec_elems, int* wpg, int* nv) {
     if (nvec <= 0) return false;
     if (nvec <= 256) { *wpg = 1; *nv = (int)((nvec + 63) / 64); return true; }
-    if (nvec <= 1024) { *wpg = 4; *nv = (int)((nvec + 255) / 256); return true; }
+    // up to 8192 channels per group in either type: 4 vectors of 8 per lane (16-bit), 8 vectors of 4 (fp32)
+    if (nvec * vec_elems <= 8192) { *wpg = 4; *nv = (int)((nvec + 255) / 256); return true; }
     return false;
 }
 
@@ -296,12 +297,13 @@ template <typename T, bool BWD>
 int launch_norm(const NormArgs& a, int64_t groups, hipStream_t st) {
     constexpr int V = GlueVec<T>::V;
     int wpg = 0, nv = 0;
-    if (!norm_shape(a.gw / V, &wpg, &nv))
-        return fail(M2_ERR_SHAPE, "rmsnorm_gated: %lld channels per group exceed the supported %d", (long long)a.gw, 1024 * V);
+    if (!norm_shape(a.gw / V, V, &wpg, &nv))
+        return fail(M2_ERR_SHAPE, "rmsnorm_gated: %lld channels per group exceed the supported 8192", (long long)a.gw);
     const dim3 grid((unsigned)ceil_div(a.rows, a.rows_per_block), (unsigned)groups);
 #define M2_NORM_CASE(W, N) if (wpg == W && nv == N) { rmsnorm_gated_kernel<T, W, N, BWD><<<grid, 256, 0, st>>>(a); return check_launch("rmsnorm_gated_kernel"); }
     M2_NORM_CASE(1, 1) M2_NORM_CASE(1, 2) M2_NORM_CASE(1, 3) M2_NORM_CASE(1, 4)
     M2_NORM_CASE(4, 2) M2_NORM_CASE(4, 3) M2_NORM_CASE(4, 4)
+    if constexpr (sizeof(T) == 4) { M2_NORM_CASE(4, 5) M2_NORM_CASE(4, 6) M2_NORM_CASE(4, 7) M2_NORM_CASE(4, 8) }
 #undef M2_NORM_CASE
     return fail(M2_ERR_SHAPE, "rmsnorm_gated: no kernel for %d waves x %d vectors", wpg, nv);
 }
@@ -474,8 +476,8 @@ extern "C" int m2_rmsnorm_gated_bwd(const m2_rmsnorm_params* p, void* stream) {
         a.rows = p->rows; a.d = p->channels; a.gw = p->channels / p->n_groups; a.eps = p->eps;
         a.rows_per_block = norm_rows_per_block(p->rows, p->n_groups, true);
         int wpg = 0, nv = 0;
-        if (!norm_shape(a.gw / V, &wpg, &nv))
-            return fail(M2_ERR_SHAPE, "rmsnorm_gated_bwd: %lld channels per group exceed the supported %d", (long long)a.gw, 1024 * V);
+        if (!norm_shape(a.gw / V, V, &wpg, &nv))
+            return fail(M2_ERR_SHAPE, "rmsnorm_gated_bwd: %lld channels per group exceed the supported 8192", (long long)a.gw);
         prows = ceil_div(p->rows, a.rows_per_block) * (wpg == 4 ? 1 : 4);
         M2_DISPATCH_DTYPE(p->dtype, T, rc = (launch_norm<T, true>(a, p->n_groups, st)));
         if (rc) return rc;

@@ -698,6 +698,11 @@ extern "C" int m2_ssd_bwd(const m2_ssd_params* p, void* stream) {
     const int V = p->dtype == M2_F32 ? 4 : 8;
     M2_REQUIRE(p->dy_stride_b % V == 0 && p->dy_stride_l % V == 0 && p->dy_stride_h % V == 0 && aligned16(p->dy), M2_ERR_ALIGN,
                "ssd_bwd: dy must be 16-byte aligned with strides that are multiples of %d elements", V);
+    // the gradients leave as 16-byte row stores
+    M2_REQUIRE(p->dx_stride_b % V == 0 && p->dx_stride_l % V == 0 && p->dx_stride_h % V == 0 && aligned16(p->dx) &&
+               p->dB_stride_b % V == 0 && p->dB_stride_l % V == 0 && p->dB_stride_g % V == 0 && aligned16(p->dB) &&
+               p->dC_stride_b % V == 0 && p->dC_stride_l % V == 0 && p->dC_stride_g % V == 0 && aligned16(p->dC), M2_ERR_ALIGN,
+               "ssd_bwd: dx, dB, dC must be 16-byte aligned with strides that are multiples of %d elements", V);
     const size_t need = m2_ssd_bwd_workspace_bytes(p);
     M2_REQUIRE(p->workspace && p->workspace_bytes >= need, M2_ERR_WORKSPACE, "ssd_bwd: workspace %zu bytes < %zu needed",
                p->workspace_bytes, need);

@@ -74,6 +74,7 @@ class RmsnormParams(C.Structure):
 SYMBOLS = {
     "m2_abi_version": (C.c_int, []),
     "m2_last_error": (C.c_char_p, []),
+    "m2_struct_layout": (C.c_int, [_i32, C.POINTER(_i64), _i32]),
     "m2_conv1d_fwd": (C.c_int, [C.POINTER(Conv1dParams), _vp]),
     "m2_conv1d_bwd_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
     "m2_conv1d_bwd": (C.c_int, [C.POINTER(Conv1dParams), _vp]),

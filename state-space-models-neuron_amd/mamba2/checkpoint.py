@@ -109,14 +109,20 @@ def _sections(key, cfg):
 
 
 def _is_replicated(key):
-    return ("norm" in key and "mixer" not in key) or "embedding" in key or key.startswith("lm_head")
+    """Block norms and the final norm are the only tensors every rank holds whole (``merge_tp_checkpoints.py:66-67``,
+    ``mamba2_inference_no_tp.py:157-158``); the embedding table and the LM head are sharded along the vocabulary like any
+    other column-parallel tensor (``ParallelEmbedding`` / ``ColumnParallelLinear``; the loaders' else-branches)."""
+    return "norm" in key and "mixer" not in key
 
 
 def shard_state_dict(state_dict, rank: int, tp: int, cfg) -> Dict[str, torch.Tensor]:
     """The slice of a full state dict that tensor-parallel rank ``rank`` of ``tp`` holds (``mamba2_inference_no_tp.py:142-165``).
-    Embedding table, LM head and block norms are kept whole (a caller sharding the vocabulary slices those itself)."""
+    Block norms are kept whole; the embedding table and the LM head are cut along the vocabulary."""
     if cfg.n_groups % tp or cfg.num_heads % tp:
         raise ValueError(f"n_groups {cfg.n_groups} and num_heads {cfg.num_heads} must be divisible by tp {tp}")
+    for k, v in state_dict.items():
+        if ("embedding" in k or k.startswith("lm_head")) and v.shape[0] % tp:
+            raise ValueError(f"{k}: vocabulary {v.shape[0]} is not divisible by tp {tp}")
     out = {}
     for k, v in state_dict.items():
         if _is_replicated(k):

@@ -1,68 +1,16 @@
 """Elementwise glue of the mixer core: softplus(dt + dt_bias) and the gated, grouped RMSNorm, forward and
 backward (``mamba2/fused_kernel.py:33-73,76-175``; torch twins ``mamba2/mamba2_mixer.py:36-38,88-105``).
 
-Three forms.  The ``*_hip`` functions call the HIP kernels (one pass over each tensor, strided rows taken in place) and
-are what the fused mixer core uses.  ``rmsnorm_gated_fn`` wraps the forward and backward kernels in an autograd function,
-for the norm modules (``MambaRMSNormGated``, the blocks' ``Mamba2RMSNorm``) and the one-token decode step.  The plain
-functions are the same math as differentiable torch device ops, for group widths the kernels do not hold in registers.
+The ``*_hip`` functions call the HIP kernels (one pass over each tensor, strided rows taken in place) and are what the
+fused mixer core uses.  ``rmsnorm_gated_fn`` wraps the forward and backward kernels in an autograd function, for the norm
+modules (``MambaRMSNormGated``, the blocks' ``Mamba2RMSNorm``) and the one-token decode step.  There is no other path:
+shapes the kernels do not take (a group wider than 8192 channels, or not a multiple of the 16-byte vector) raise.
 """
 import ctypes as C
 
 import torch
-import torch.nn.functional as F
 
 from . import _lib
-
-SOFTPLUS_THRESHOLD = 10.0      # mamba2_mixer.py:36
-
-
-def softplus_bias(dt, dt_bias):
-    """softplus(dt + dt_bias) with the reference's threshold form; result in the dtype of dt."""
-    v = dt.float() + dt_bias.float()
-    return torch.where(v < SOFTPLUS_THRESHOLD, torch.log1p(torch.exp(torch.clamp(v, max=SOFTPLUS_THRESHOLD))), v).to(dt.dtype)
-
-
-def softplus_bias_bwd(dt, dt_bias, d_out, out_d_in=None):
-    """d_in = d_out * sigmoid(dt + dt_bias) (1 above the threshold); returns d_bias (h) fp32 (fused_kernel.py:68-72)."""
-    v = dt.float() + dt_bias.float()
-    d_in = d_out.float() * torch.where(v < SOFTPLUS_THRESHOLD, torch.sigmoid(v), torch.ones_like(v))
-    if out_d_in is not None:
-        out_d_in.copy_(d_in)
-    return d_in.sum(dim=tuple(range(d_in.dim() - 1)))
-
-
-def rmsnorm_gated(x, z, weight, n_groups, eps, out_dtype=None):
-    """h = x * silu(z); per group of d/g contiguous channels out = h * rsqrt(mean h^2 + eps) * w, in fp32."""
-    h = x.float()
-    if z is not None:
-        h = h * F.silu(z.float())
-    shp = h.shape
-    hg = h.reshape(*shp[:-1], n_groups, shp[-1] // n_groups)
-    hg = hg * torch.rsqrt(hg.pow(2).mean(-1, keepdim=True) + eps)
-    out = weight.float() * hg.reshape(shp)
-    return out if out_dtype is None else out.to(out_dtype)
-
-
-def rmsnorm_gated_bwd(x, z, weight, d_out, n_groups, eps, out_dz=None):
-    """Returns (dx, dw fp32); dz is written into ``out_dz`` (fused_kernel.py:159-171)."""
-    xf, zf, g = x.float(), z.float(), d_out.float()
-    sig = torch.sigmoid(zf)
-    gate = zf * sig
-    h = xf * gate
-    shp = h.shape
-    G = n_groups
-    hg = h.reshape(*shp[:-1], G, shp[-1] // G)
-    var = hg.pow(2).mean(-1, keepdim=True) + eps
-    rinv = torch.rsqrt(var)
-    gw = (g * weight.float()).reshape(hg.shape)
-    cf = (hg * gw).mean(-1, keepdim=True) / var
-    d_h = (rinv * (gw - cf * hg)).reshape(shp)
-    dw = (g * (hg * rinv).reshape(shp)).sum(dim=tuple(range(g.dim() - 1)))
-    dx = (d_h * gate).to(x.dtype)
-    dz = d_h * xf * (sig * (1 + zf * (1 - sig)))
-    if out_dz is not None:
-        out_dz.copy_(dz)
-    return dx, dw
 
 
 # --------------------------------------------------------------------------------------------- HIP kernels
@@ -230,8 +178,8 @@ def norm_kernel_ok(x, n_groups):
     if x.dtype not in (torch.float32, torch.bfloat16) or n_groups < 1 or x.shape[-1] % n_groups:
         return False
     gw = x.shape[-1] // n_groups
-    vec, cap = (8, 8192) if x.dtype == torch.bfloat16 else (4, 4096)
-    return gw % vec == 0 and 0 < gw <= cap
+    vec = 8 if x.dtype == torch.bfloat16 else 4
+    return gw % vec == 0 and 0 < gw <= 8192
 
 
 class RmsnormGated(torch.autograd.Function):
@@ -252,8 +200,11 @@ class RmsnormGated(torch.autograd.Function):
 
 def rmsnorm_gated_fn(x, z, weight, n_groups, eps, out_dtype=None):
     """Differentiable gated grouped RMSNorm; output fp32 unless ``out_dtype`` says the dtype of x.
-    Shapes outside the kernels' limits go through the torch device ops (same math, autograd builds the backward)."""
+    Raises ValueError for shapes outside the kernels' limits."""
     _lib.require_gpu(x, z, weight)
-    if not norm_kernel_ok(x, n_groups) or (z is not None and z.dtype != x.dtype):
-        return rmsnorm_gated(x, z, weight, n_groups, eps, out_dtype=out_dtype)
+    if not norm_kernel_ok(x, n_groups):
+        raise ValueError(f"rmsnorm_gated: {x.shape[-1]} channels in {n_groups} groups, dtype {x.dtype}: a group must be a "
+                         "multiple of 16 bytes and at most 8192 channels wide, in float32 or bfloat16")
+    if z is not None and z.dtype != x.dtype:
+        raise ValueError("rmsnorm_gated: z must have the dtype of x")
     return RmsnormGated.apply(x, z, weight, n_groups, eps, out_dtype)

@@ -24,7 +24,7 @@ def test_header_symbols_exported_and_bound(lib):
         assert hasattr(lib, s), f"{s} declared in the header but not exported"
         assert s in _lib.SYMBOLS, f"{s} has no ctypes prototype"
     assert sorted(_lib.SYMBOLS) == syms
-    assert lib.m2_abi_version() == 3
+    assert lib.m2_abi_version() == 4
 
 
 def test_struct_sizes_match_header():
@@ -45,6 +45,19 @@ def test_struct_sizes_match_header():
             names.append(first)
             names += [q.strip().lstrip("*") for q in parts[1:]]
         assert names == [f[0] for f in pyc._fields_], cname
+
+
+def test_struct_layout_matches_library(lib):
+    # size and every field offset of the ctypes mirrors against what the compiled library reports
+    from mamba2 import _lib
+    for which, pyc in enumerate((_lib.Conv1dParams, _lib.SsdParams, _lib.DecodeParams, _lib.RmsnormParams)):
+        buf = (ctypes.c_int64 * 128)()
+        n = lib.m2_struct_layout(which, buf, 128)
+        assert n == 1 + len(pyc._fields_), pyc.__name__
+        assert buf[0] == ctypes.sizeof(pyc), pyc.__name__
+        for i, (fname, _) in enumerate(pyc._fields_):
+            assert buf[1 + i] == getattr(pyc, fname).offset, f"{pyc.__name__}.{fname}"
+    assert lib.m2_struct_layout(9, (ctypes.c_int64 * 4)(), 4) == -1
 
 
 def test_validation_before_any_device_call(lib):

@@ -66,10 +66,50 @@ def test_tp_shard_then_merge_is_identity(tp):
         assert torch.equal(s1[k + "conv1d.weight"], torch.cat([cw[128:256], cw[256 + 32:256 + 64], cw[320 + 32:320 + 64]]))
         assert torch.equal(s1[k + "A_log"], sd[k + "A_log"][2:]) and torch.equal(s1[k + "norm.weight"], sd[k + "norm.weight"][128:])
         assert torch.equal(s1["backbone.layers.0.norm.weight"], sd["backbone.layers.0.norm.weight"])      # replicated
+        # the embedding table and the LM head are cut along the vocabulary (mamba2_inference_no_tp.py:159-162)
+        v = sd["backbone.embeddings.weight"].shape[0]
+        assert torch.equal(s1["backbone.embeddings.weight"], sd["backbone.embeddings.weight"][v // 2:])
+        assert torch.equal(s1["lm_head.weight"], sd["lm_head.weight"][v // 2:])
     merged = merge_tp_state_dicts(shards, cfg)
     assert merged.keys() == sd.keys() and all(torch.equal(merged[n], sd[n]) for n in sd)
     with pytest.raises(ValueError):
         shard_state_dict(sd, 0, 3, cfg)
+
+
+def test_merge_shards_built_the_trainers_way():
+    """Shards cut the way the reference's loader cuts them (mamba2_inference_no_tp.py:142-165, written out here
+    independently of shard_state_dict: one group per rank, n_groups == tp as the trainer forces, train.py:44) merge back
+    into the full state dict, vocabulary-split table and head included (merge_tp_checkpoints.py:6-72)."""
+    from mamba2.checkpoint import merge_tp_state_dicts, shard_state_dict
+    cfg = _cfg(vocab_size=48)
+    sd = _random_model(cfg, seed=5).state_dict()
+    tp = cfg.n_groups
+    d_inner, gn, h = cfg.num_heads * cfg.head_dim, cfg.n_groups * cfg.state_size, cfg.num_heads
+
+    def cut(v, sections, r):
+        return torch.cat([torch.split(part, part.shape[0] // tp, dim=0)[r] for part in torch.split(v, sections, dim=0)], dim=0)
+
+    shards = []
+    for r in range(tp):
+        sh = {}
+        for k, v in sd.items():
+            if k.endswith("out_proj.weight"):
+                sh[k] = torch.split(v, v.shape[1] // tp, dim=1)[r]
+            elif "conv1d" in k:
+                sh[k] = cut(v, [d_inner, gn, gn], r)
+            elif k.endswith("in_proj.weight"):
+                sh[k] = cut(v, [d_inner, d_inner, gn, gn, h], r)
+            elif "norm" in k and "mixer" not in k:
+                sh[k] = v
+            else:
+                sh[k] = torch.split(v, v.shape[0] // tp, dim=0)[r]
+        shards.append(sh)
+    assert shards[0]["backbone.embeddings.weight"].shape[0] == 48 // tp and shards[1]["lm_head.weight"].shape[0] == 48 // tp
+    merged = merge_tp_state_dicts(shards, cfg)
+    assert merged.keys() == sd.keys() and all(torch.equal(merged[n], sd[n]) for n in sd)
+    for r in range(tp):
+        mine = shard_state_dict(sd, r, tp, cfg)
+        assert all(torch.equal(mine[n], shards[r][n]) for n in sd), r
 
 
 def test_load_state_spaces_and_codestral_directories(tmp_path):

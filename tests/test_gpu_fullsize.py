@@ -125,9 +125,11 @@ def test_mixer_layer_full_shape_batch_rows_independent(hidden, heads, groups, b,
     x1 = x.detach()[b - 1:].clone().requires_grad_(True)
     y1 = mix(x1)
     y1.backward(dy[b - 1:])
-    # the projections may pick different GEMM tiles for the one-row batch: the bf16 bar, not bit equality
-    assert rel_rms_err(y1, y.detach()[b - 1:].float(), roundings=2) < 2e-2
-    assert rel_rms_err(x1.grad, x.grad[b - 1:].float(), roundings=2) < 2e-2
+    # the projections may pick different GEMM tiles for the one-row batch, so this compares two bf16 computations, each
+    # within 2e-2 x RMS of the exact result: triangle inequality, and a tight relative-L2 bound
+    for a_, b_ in ((y1, y.detach()[b - 1:]), (x1.grad, x.grad[b - 1:])):
+        assert rel_rms_err(a_.float(), b_.float()) < 4e-2
+        assert ((a_.float() - b_.float()).norm() / b_.float().norm()).item() < 5e-3
 
 
 def test_model_step_full_width_two_layers():

@@ -1,0 +1,105 @@
+"""GPU: parity against the fp64 CPU oracle AT the benchmark configurations (through the C ABI).
+
+* c1  SSD fwd+bwd, b4 l2048 h80 p64 n128 g1, bf16: y, final state, dx, ddt, dA, dB, dC, dD;
+* c3  the 7B layer's SSD shape, b2 l4096 h128 p64 n128 g8, bf16: the same eight tensors;
+* c2  conv1d + SiLU fwd+bwd, b4 l2048 C5376, bf16: y, dx, dw, db;
+* c4  one decode step at batch 128 (h80 p64 n128 C5376, W = 3, the real conv with SiLU), then the 64 stacked layers of one
+      step, every layer with its own states, each checked against the oracle.
+
+The bar is the stated one: fp32 results max|err| / max|ref| <= 1e-4; bf16 computations max|err| <= 2e-2 x RMS(ref) on the
+RAW error, plus, for a tensor stored in bf16, what storing the exact value costs (conftest.rel_rms_err; every raw figure
+is logged).  Inputs follow the reference's parity script (mamba2_kernel.py:555-564) as the configurations state them.
+"""
+import math
+
+import pytest
+import torch
+
+from conftest import rel_err, rel_rms_err
+from oracle.conv import conv1d_grads_ref, make_conv_inputs
+from oracle.decode import decode_step_ref
+from oracle.ssd import make_ssd_inputs, ssd_grads_ref
+
+pytestmark = [pytest.mark.gpu, pytest.mark.timeout(900)]
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("b,l,h,p,n,g", [(4, 2048, 80, 64, 128, 1), (2, 4096, 128, 64, 128, 8)], ids=["c1", "c3"])
+def test_ssd_fwd_bwd_against_oracle_full_size(b, l, h, p, n, g):
+    from mamba2.mamba2_kernel import mamba2_kernel
+    d = make_ssd_inputs(b, l, h, p, n, g, seed=0, dtype=torch.bfloat16)
+    torch.set_num_threads(min(16, torch.get_num_threads()))
+    ref = ssd_grads_ref(*(d[k].double() for k in ("dt", "A", "X", "B", "C", "D", "dy")))
+    lv = {k: d[k].to(DEV).requires_grad_(True) for k in ("dt", "A", "X", "B", "C", "D")}
+    y, S = mamba2_kernel(lv["dt"], lv["A"], lv["X"], lv["B"], lv["C"], lv["D"], return_final_state=True)
+    y.backward(d["dy"].to(DEV))
+    assert y.dtype == torch.bfloat16 and S.dtype == torch.float32
+    got = {"y": y.detach(), "final_state": S.detach(), "dX": lv["X"].grad, "ddt": lv["dt"].grad, "dA": lv["A"].grad,
+           "dB": lv["B"].grad, "dC": lv["C"].grad, "dD": lv["D"].grad}
+    bad = {}
+    for k, v in got.items():
+        # y, dx, ddt, dB, dC leave in bf16; the final state and dA are fp32 sums of MFMA products whose operands (the
+        # decay-weighted dt x rows) were rounded to bf16: the error of an element is proportional to its own magnitude
+        e = rel_rms_err(v.cpu(), ref[k], name=k, bf16_operands=True)
+        l2 = ((v.double().cpu() - ref[k]).norm() / ref[k].norm()).item()
+        if not (e < 2e-2 and l2 < 1e-2):
+            bad[k] = (e, l2)
+    assert not bad, bad
+
+
+def test_conv_fwd_bwd_against_oracle_c2():
+    from mamba2.conv1d_grouped import conv1d_backward, conv1d_forward
+    d = make_conv_inputs(4, 2048, 5376, 4, seed=0, dtype=torch.bfloat16)
+    y_ref, dx_ref, dw_ref, db_ref = conv1d_grads_ref(d["x"].double(), d["w"].double(), d["bias"].double(), d["dy"].double(), "silu")
+    x, w, bias, dy = (d[k].to(DEV) for k in ("x", "w", "bias", "dy"))
+    y = conv1d_forward(x, w, bias, "silu", channels_last=True)
+    dx, dw, db = conv1d_backward(x, w, bias, dy, "silu", channels_last=True)
+    assert rel_rms_err(y.cpu(), y_ref, name="y") < 2e-2
+    assert rel_rms_err(dx.cpu(), dx_ref, name="dx") < 2e-2
+    # dw, db: sums over 8192 tokens, reduced in fp32 and stored in the parameter type
+    assert rel_rms_err(dw.cpu(), dw_ref, name="dw") < 2e-2
+    assert rel_rms_err(db.cpu(), db_ref, name="db") < 2e-2
+    assert ((dw.double().cpu() - dw_ref).norm() / dw_ref.norm()).item() < 5e-3
+
+
+def _decode_layer_inputs(gen, b, h, p, n, g, W, k):
+    """One layer's token inputs and states, drawn on the device (the states of 64 layers are 21.5 GB): x ~ N(0,1) (B, C
+    columns / sqrt(n)), dt = exp(U(log 1e-3, log 1e-1)), S ~ N(0, 0.1) fp32, conv state ~ N(0,1) bf16."""
+    d_inner, Cx = h * p, h * p + 2 * g * n
+    xBC = torch.randn(b, 1, Cx, device=DEV, generator=gen)
+    xBC[:, :, d_inner:] /= math.sqrt(n)
+    conv_state = torch.randn(b, Cx, W, device=DEV, generator=gen).to(torch.bfloat16)
+    S = 0.1 * torch.randn(b, h, p, n, device=DEV, generator=gen)
+    dt = torch.exp(torch.empty(b, 1, h, device=DEV).uniform_(math.log(1e-3), math.log(1e-1), generator=gen))
+    return xBC.to(torch.bfloat16), conv_state, S, dt.to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("layers", [1, 64])
+def test_decode_step_against_oracle_c4(layers):
+    from mamba2.mamba2_kernel_inference import mamba2_kernel_inference
+    b, h, p, n, g, W, k = 128, 80, 64, 128, 1, 3, 4
+    Cx = h * p + 2 * g * n
+    gen = torch.Generator(device=DEV).manual_seed(11)
+    cg = torch.Generator().manual_seed(12)
+    A = -torch.exp(torch.empty(h).uniform_(0.0, math.log(16.0), generator=cg))
+    D = torch.ones(h)
+    w = (torch.rand(Cx, k, generator=cg) - 0.5).to(torch.bfloat16)
+    bias = (torch.rand(Cx, generator=cg) - 0.5).to(torch.bfloat16)
+    Ad, Dd, wd, bd = (t.to(DEV) for t in (A, D, w, bias))
+    state = [_decode_layer_inputs(gen, b, h, p, n, g, W, k) for _ in range(layers)]
+    before = [tuple(t.cpu() for t in s) for s in state] if layers == 1 else None
+    outs = []
+    for i, (xBC, conv_state, S, dt) in enumerate(state):
+        keep = (xBC.cpu(), conv_state.cpu(), S.cpu(), dt.cpu()) if before is None else before[i]
+        y, cs, S2 = mamba2_kernel_inference(xBC, conv_state, wd, bd, S, dt, Ad, Dd, n_groups=g)
+        assert cs.data_ptr() == conv_state.data_ptr() and S2.data_ptr() == S.data_ptr()      # in place
+        outs.append((keep, y))
+    torch.cuda.synchronize()
+    for i, ((xBC, conv_state, S, dt), y) in enumerate(outs):
+        y_ref, cs_ref, S_ref = decode_step_ref(xBC.double(), conv_state.double(), w.double(), bias.double(), S.double(),
+                                               dt.double(), A.double(), D.double(), n_groups=g)
+        # the conv state is a shift of stored values: bit-exact; the state update is fp32 arithmetic on fp32 state
+        assert torch.equal(state[i][1].cpu().double(), cs_ref), i
+        assert rel_err(state[i][2].cpu(), S_ref) < 1e-4, i
+        # y leaves in bf16
+        assert rel_rms_err(y.cpu(), y_ref, name=f"y[layer {i}]" if i < 2 else None) < 2e-2, i

@@ -63,8 +63,6 @@ NORM_SHAPES = [
 @pytest.mark.parametrize("gated", [True, False])
 def test_rmsnorm_gated_fwd_bwd(dtype, rows, d, g, gated):
     from mamba2 import glue
-    if dtype == torch.float32 and d // g > 4096:
-        pytest.skip("fp32 groups are limited to 4096 channels")
     eps = 1e-5
     x = _rand((*rows, d), dtype, 11)
     z = _rand((*rows, d), dtype, 12) if gated else None
@@ -88,9 +86,9 @@ def test_rmsnorm_gated_fwd_bwd(dtype, rows, d, g, gated):
     # dx, dz are stored in the input type.  h = x silu(z) is heavy-tailed (elements beyond 10 RMS), and a bf16 value just
     # above a power of two is off by up to 2^-8 of itself from storage alone: roundings=2 discounts that worst case
     # instead of the 2^-9 best case, the arithmetic (fp32 throughout) must stay inside the tolerance
-    assert rel_rms_err(dx.cpu(), xd.grad, roundings=2) < TOL[dtype]
+    assert rel_rms_err(dx.cpu(), xd.grad) < TOL[dtype]
     if gated:
-        assert rel_rms_err(dz.cpu(), zd.grad, roundings=2) < TOL[dtype]
+        assert rel_rms_err(dz.cpu(), zd.grad) < TOL[dtype]
     else:
         assert dz is None
     # dw is an fp32 sum over the rows of products of the (bf16) inputs: the inputs are exact, the sum is not rounded to bf16

@@ -216,7 +216,7 @@ def test_ssd_softplus_folded_into_scan(dtype, b, l, h, p, n, g):
         else:
             # stored in bf16, and heavy-tailed here (the tokens with step sizes beyond the threshold): a bf16 value just
             # above a power of two is off by up to 2^-8 of itself from storage alone, which roundings=2 discounts
-            assert rel_rms_err(ddt.cpu(), dt_raw.grad, roundings=2) < tol
+            assert rel_rms_err(ddt.cpu(), dt_raw.grad) < tol
         # a signed sum over all b * l tokens of ddt terms that are each within the tolerance: a few times the element bound
         assert err(dbias.cpu(), bias_d.grad) < (5e-4 if dtype == torch.float32 else tol)
         assert err(dX.cpu(), lv["X"].grad) < tol
