@@ -166,6 +166,18 @@ typedef struct m2_decode_params {
 size_t m2_decode_workspace_bytes(int64_t batch, int64_t nheads, int64_t headdim, int64_t dstate, int64_t ngroups);
 int m2_decode_step(const m2_decode_params* p, void* stream);
 
+/* m2_decode_step for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc): the same kernels, same inputs and outputs, but the step's scratch -- the activated conv output,
+ * batch x (nheads*headdim + 2*ngroups*dstate) floats -- lives in a 4 MiB array inside the library's device image
+ * instead of a caller workspace; p->workspace and p->workspace_bytes are ignored.  No counterpart in the reference
+ * (its decode kernel allocates fresh outputs per call, mamba2_kernel_inference.py:114-116).
+ *   - limit: batch x conv channels <= 1 048 576 (batch 195 at the 2.7B width); beyond it M2_ERR_WORKSPACE.
+ *   - allocates nothing; the array's device address is looked up on the first call per device (make that first call
+ *     outside a graph capture).  Each GPU holds its own 4 MiB copy until the process ends.
+ *   - all calls on one GPU share that array: calls that overlap on one GPU (two streams, two threads) race; calls on
+ *     one stream, or otherwise ordered, are safe.  Nothing in it has to start at zero (every call overwrites what it reads). */
+int m2_decode_step_static(const m2_decode_params* p, void* stream);
+
 /* ------------------------------------------------------------------ mixer glue
  * The elementwise passes between the conv, the scan and the output projection
  * (mamba2/fused_kernel.py:33-47 softplus_with_bias, :50-73 softplus_with_bias_bwd,

@@ -14,6 +14,8 @@
 //   decode_ssm_kernel    one workgroup per (head, batch); a group of lanes owns one state row p and walks
 //                        n with 16-byte accesses, so a wave issues whole 128-byte-or-wider lines and every
 //                        state element is touched by exactly one thread (in-place update is race free).
+#include <mutex>
+
 #include "common.hpp"
 
 namespace m2 {
@@ -203,9 +205,65 @@ extern "C" size_t m2_decode_workspace_bytes(int64_t batch, int64_t nheads, int64
     return (size_t)(batch * (nheads * headdim + 2 * ngroups * dstate)) * sizeof(float) + 16;
 }
 
+namespace m2 {
+namespace {
+
+// Scratch of the entry point that allocates nothing: the activated conv output of one step, held in the library's own
+// device image (every GPU the library runs on holds its own copy until the process ends).
+constexpr size_t kStaticScratchFloats = (size_t)1 << 20;          // 4 MiB: batch x conv channels <= 1 048 576
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+float* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the CURRENT device, looked up once per device (the array's name is only a host-side
+// handle: kernels and copies get this pointer).
+int static_scratch(float** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return fail(M2_ERR_LAUNCH, "decode_step_static: hipGetDevice failed or device index %d out of range", dev);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            return fail(M2_ERR_LAUNCH, "decode_step_static: hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = static_cast<float*>(ptr);
+    }
+    *out = g_scratch_ptr[dev];
+    return M2_OK;
+}
+
+int decode_step_impl(const m2_decode_params* p, float* act, size_t act_bytes, const char* who, void* stream);
+
+}  // namespace
+}  // namespace m2
+
 extern "C" int m2_decode_step(const m2_decode_params* p, void* stream) {
     using namespace m2;
     M2_REQUIRE(p, M2_ERR_NULL, "decode_step: params is NULL");
+    return decode_step_impl(p, static_cast<float*>(p->workspace), p->workspace_bytes, "decode_step", stream);
+}
+
+extern "C" int m2_decode_step_static(const m2_decode_params* p, void* stream) {
+    using namespace m2;
+    M2_REQUIRE(p, M2_ERR_NULL, "decode_step_static: params is NULL");
+    const int64_t Cx = p->nheads * p->headdim + 2 * p->ngroups * p->dstate;
+    // sizes beyond the built-in scratch are refused here; every other check is the shared one below
+    M2_REQUIRE(p->batch <= 0 || Cx <= 0 || (uint64_t)Cx <= kStaticScratchFloats / (uint64_t)p->batch, M2_ERR_WORKSPACE,
+               "decode_step_static: batch %lld x %lld conv channels exceed the built-in scratch of %zu floats; use m2_decode_step with a workspace",
+               (long long)p->batch, (long long)Cx, kStaticScratchFloats);
+    float* act = nullptr;
+    const int rc = static_scratch(&act);
+    if (rc) return rc;
+    return decode_step_impl(p, act, kStaticScratchFloats * sizeof(float), "decode_step_static", stream);
+}
+
+namespace m2 {
+namespace {
+
+int decode_step_impl(const m2_decode_params* p, float* act, size_t act_bytes, const char* who, void* stream) {
     M2_REQUIRE(p->dtype == M2_F32 || p->dtype == M2_BF16, M2_ERR_DTYPE, "decode_step: bad dtype %d", p->dtype);
     M2_REQUIRE(p->param_dtype == M2_F32 || p->param_dtype == M2_BF16, M2_ERR_DTYPE, "decode_step: bad param dtype %d", p->param_dtype);
     M2_REQUIRE(p->batch >= 0 && p->nheads >= 0 && p->headdim >= 1 && p->dstate >= 1, M2_ERR_SHAPE, "decode_step: bad dimension");
@@ -219,11 +277,9 @@ extern "C" int m2_decode_step(const m2_decode_params* p, void* stream) {
     M2_REQUIRE(p->W == 0 || p->conv_state, M2_ERR_NULL, "decode_step: conv_state is required");
     const int64_t Cx = p->nheads * p->headdim + 2 * p->ngroups * p->dstate;
     const size_t need = (size_t)(p->batch * Cx) * sizeof(float);
-    M2_REQUIRE(p->workspace && p->workspace_bytes >= need, M2_ERR_WORKSPACE, "decode_step: workspace %zu bytes < %zu needed",
-               p->workspace_bytes, need);
-    M2_REQUIRE(aligned16(p->workspace) && aligned16(p->S), M2_ERR_ALIGN, "decode_step: workspace and S must be 16-byte aligned");
+    M2_REQUIRE(act && act_bytes >= need, M2_ERR_WORKSPACE, "%s: workspace %zu bytes < %zu needed", who, act_bytes, need);
+    M2_REQUIRE(aligned16(act) && aligned16(p->S), M2_ERR_ALIGN, "%s: workspace and S must be 16-byte aligned", who);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    float* act = static_cast<float*>(p->workspace);
     const int vec = (p->dstate % 4 == 0 && (p->nheads * p->headdim) % 4 == 0 && Cx % 4 == 0) ? 4 : 1;
     int GL = 1;
     while (GL < 64 && GL < p->dstate / vec) GL <<= 1;
@@ -264,3 +320,6 @@ extern "C" int m2_decode_step(const m2_decode_params* p, void* stream) {
     });
     return M2_OK;
 }
+
+}  // namespace
+}  // namespace m2

@@ -85,6 +85,7 @@ SYMBOLS = {
     "m2_ssd_bwd": (C.c_int, [C.POINTER(SsdParams), _vp]),
     "m2_decode_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64]),
     "m2_decode_step": (C.c_int, [C.POINTER(DecodeParams), _vp]),
+    "m2_decode_step_static": (C.c_int, [C.POINTER(DecodeParams), _vp]),
     "m2_softplus_bias_fwd": (C.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _i64, _i32, _vp]),
     "m2_softplus_bias_bwd_workspace_bytes": (_sz, [_i64, _i64]),
     "m2_softplus_bias_bwd": (C.c_int, [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _sz, _i64, _i64, _i32, _vp]),
