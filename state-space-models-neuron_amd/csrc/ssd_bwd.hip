@@ -523,7 +523,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         sa.ldtab = w.ldtab; sa.Mt = w.Ct; sa.init = p->d_final_state; sa.prev = w.dprev; sa.final_out = p->d_initial_state;
         sa.sprev = w.prev; sa.dlam = w.dlam;
         sa.seqlen = p->seqlen; sa.nheads = p->nheads; sa.ngroups = p->ngroups; sa.nchunks = nc;
-        k<<<dim3((unsigned)(p->nheads * state_pass_nsplit<N>()), (unsigned)p->batch), state_pass_threads<N>(), sm, st>>>(sa);
+        k<<<dim3((unsigned)(p->nheads * kStatePassSplit), (unsigned)p->batch), state_pass_threads<N>(), sm, st>>>(sa);
         if ((rc = check_launch("ssd state_pass16_kernel<reverse>"))) return rc;
     } else
     {   // fp32: local dS contributions (reuses the `local` region), then the reverse recurrence

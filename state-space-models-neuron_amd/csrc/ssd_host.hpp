@@ -195,7 +195,7 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
         sa.ldtab = w.ldtab; sa.Mt = w.Bt; sa.init = p->initial_state; sa.prev = w.prev; sa.final_out = final_out;
         sa.sprev = nullptr; sa.dlam = nullptr;
         sa.seqlen = p->seqlen; sa.nheads = p->nheads; sa.ngroups = p->ngroups; sa.nchunks = nc;
-        k<<<dim3((unsigned)(p->nheads * state_pass_nsplit<N>()), (unsigned)p->batch), state_pass_threads<N>(), sm, st>>>(sa);
+        k<<<dim3((unsigned)(p->nheads * kStatePassSplit), (unsigned)p->batch), state_pass_threads<N>(), sm, st>>>(sa);
         return check_launch("ssd state_pass16_kernel");
     } else {
         // fp32 operands: per-chunk contributions (fp32, workspace), then the recurrence over the chunks

@@ -8,8 +8,10 @@
 //  With DLAM == false the reverse pass leaves dlam to ssd_bwd16_kernel, which has both tiles in LDS anyway, and does
 //  not read sprev at all.)
 //
-// grid (nheads * NSPLIT, batch), 2 x NWG waves; a workgroup owns N / NSPLIT columns of the [P][N] state, wave w rows
-// [ (w & 1) P/2, +P/2 ) x one NWG-th of those columns, as 32x32 MFMA accumulator blocks.  Per chunk the MFMA computes  X_scaled^T [P x kQ] * M [kQ x N]:
+// grid (nheads * 2, batch), N / 32 waves; a workgroup owns one half of the ROWS of the [P][N] state (P / 2 head channels, all
+// N columns), wave w the columns [32 w, +32) of them, as 32x32 MFMA accumulator blocks: only that half of the x / dy columns
+// is loaded, scaled and staged, so the two workgroups of a head share no work.  Per chunk the MFMA computes
+// X_scaled^T [P/2 x kQ] * M [kQ x N]:
 //   * M (B or C of the group) comes from the transposed tiles that prep_kernel wrote in MFMA operand order: a wave's
 //     B-operand fragment is one contiguous KiB of global memory, loaded straight into registers at the top of the
 //     chunk's iteration (the tile is shared by all heads of the group and stays in L2);
@@ -34,49 +36,42 @@ struct StatePassArgs {
     int64_t seqlen, nheads, ngroups, nchunks;
 };
 
-// workgroups per (batch, head): each takes N / NSPLIT state columns (more, smaller workgroups: the chunk loop is a
-// chain of dependent memory round trips, and only other resident waves can fill its gaps)
-#ifndef M2_SP_NSPLIT
-#define M2_SP_NSPLIT(N) ((N) / 64)
-#endif
-#ifndef M2_SP_NWG
-#define M2_SP_NWG(N) 2
-#endif
-template <int N> constexpr int state_pass_nsplit() { return M2_SP_NSPLIT(N); }
-// waves per workgroup along the state columns (times two along the rows)
-template <int N> constexpr int state_pass_nwg() { return M2_SP_NWG(N); }
-template <int N> constexpr int state_pass_threads() { return 2 * state_pass_nwg<N>() * 64; }
+// workgroups per (batch, head): each takes half of the state rows (more, smaller workgroups: the chunk loop is a chain of
+// dependent memory round trips, and only other resident waves can fill its gaps)
+constexpr int kStatePassSplit = 2;
+// one wave per 32 state columns
+template <int N> constexpr int state_pass_threads() { return (N / 32) * 64; }
 template <int P, int N>
 constexpr size_t state_pass_smem() {
-    return (size_t)2 * kQ * P * 2 + (size_t)2 * state_pass_nwg<N>() * (P / 2) * (N / state_pass_nsplit<N>() / state_pass_nwg<N>() + 8) * 2;
+    return (size_t)2 * kQ * (P / 2) * 2 + (size_t)(N / 32) * (P / 2) * (32 + 8) * 2;
 }
 
 template <typename T, int P, int N, bool REVERSE, bool DLAM = REVERSE>
 __global__ void __launch_bounds__(state_pass_threads<N>(), (P == 64 ? (DLAM ? 2 : 3) : (DLAM ? 1 : 2)))
 state_pass16_kernel(const StatePassArgs a) {
     static_assert(sizeof(T) == 2, "16-bit operands only");
-    constexpr int NSPLIT = state_pass_nsplit<N>();
-    constexpr int NWG = state_pass_nwg<N>(), THREADS = state_pass_threads<N>();
-    constexpr int NW = N / NSPLIT / NWG;               // state columns per wave
-    static_assert(NW % 32 == 0 && 2 * NWG * NSPLIT <= kDlamParts, "wave blocks / dlam slots");
-    constexpr int PBW = P / 64, NBW = NW / 32;         // 32x32 blocks per wave
-    constexpr int SPR_X = P / 8;                       // 16-byte slots per x row
+    constexpr int NWAVES = N / 32, THREADS = state_pass_threads<N>();
+    constexpr int PH = P / 2;                          // state rows (head channels) of this workgroup
+    constexpr int NW = 32;                             // state columns per wave
+    static_assert(kStatePassSplit * NWAVES <= kDlamParts, "dlam slots");
+    constexpr int PBW = PH / 32, NBW = 1;              // 32x32 blocks per wave
+    constexpr int SPR_X = PH / 8;                      // 16-byte slots per staged x row
     constexpr int NXR = kQ * SPR_X / THREADS;              // x pieces per thread per chunk
     constexpr int LDO = NW + 8;
     constexpr int LPR = NW / 8;                   // lanes per row of this wave's state block (8 elements each)
     constexpr int RPP = 64 / LPR;                      // rows per store pass
     constexpr int NSP = (P / 2) / RPP;                 // store passes
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    T* sX = reinterpret_cast<T*>(smem_raw);                                 // [2][kQ][P], slots swizzled inside each row
-    T* sO = sX + 2 * kQ * P;                                                // [waves][P / 2][LDO]
+    T* sX = reinterpret_cast<T*>(smem_raw);                                 // [2][kQ][P / 2], slots swizzled inside each row
+    T* sO = sX + 2 * kQ * PH;                                               // [waves][P / 2][LDO]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 31, half = lane >> 5;
-    const int pw = wave & 1, nw = wave >> 1;
+    const int pw = (int)(blockIdx.x / a.nheads);       // which half of the rows
     // the workgroups of one head are nheads apart in the grid: with a head count that is a multiple of 8 they land on the
     // same XCD and share the head's rows in its L2
     const int64_t h = blockIdx.x % a.nheads, b = blockIdx.y;
-    const int n0 = (int)(blockIdx.x / a.nheads) * (N / NSPLIT) + nw * NW;      // first state column of this wave
+    const int n0 = wave * NW;                          // first state column of this wave
     const int64_t g = h / (a.nheads / a.ngroups);
     const int64_t bh = b * a.nheads + h;
     const int64_t nc = a.nchunks;
@@ -115,7 +110,7 @@ state_pass16_kernel(const StatePassArgs a) {
     auto load_ahead = [&](int64_t c, Ahead& s) {
         const int64_t t0 = c * kQ;
         const uint32_t last = (uint32_t)(((a.seqlen - t0) < kQ ? (a.seqlen - t0) : kQ) - 1);      // last valid row
-        const char* xp = reinterpret_cast<const char*>(static_cast<const T*>(a.X) + b * a.X_sb + t0 * a.X_sl + h * a.X_sh);
+        const char* xp = reinterpret_cast<const char*>(static_cast<const T*>(a.X) + b * a.X_sb + t0 * a.X_sl + h * a.X_sh + pw * PH);
         const float* tab = a.ldtab + (bh * nc + c) * (2 * kQ);
         s.lam = tab[kQ - 1];
 #pragma unroll
@@ -160,7 +155,7 @@ state_pass16_kernel(const StatePassArgs a) {
             case 2: __builtin_amdgcn_s_setprio(1); break;
             default: __builtin_amdgcn_s_setprio(0); break;
         }
-        T* cX = sX + buf * (kQ * P);
+        T* cX = sX + buf * (kQ * PH);
         __builtin_amdgcn_sched_barrier(0);      // keep this chunk's loads out of the previous chunk's MFMA phase (registers)
         load_same(c);
         // the values loaded one chunk ahead become visible to the optimiser here and no earlier: otherwise their
@@ -212,9 +207,10 @@ state_pass16_kernel(const StatePassArgs a) {
         if (DLAM) {
             dot = warp_sum(dot);
             if (lane == 0) {
-                const int slot = (int)(blockIdx.x / a.nheads) * (2 * NWG) + wave;
+                const int slot = pw * NWAVES + wave;
                 a.dlam[(bh * nc + c) * kDlamParts + slot] = dec * dot;
-                if (2 * NWG * NSPLIT < kDlamParts && slot + 2 * NWG * NSPLIT < kDlamParts) a.dlam[(bh * nc + c) * kDlamParts + slot + 2 * NWG * NSPLIT] = 0.f;
+                if (kStatePassSplit * NWAVES < kDlamParts && slot + kStatePassSplit * NWAVES < kDlamParts)
+                    a.dlam[(bh * nc + c) * kDlamParts + slot + kStatePassSplit * NWAVES] = 0.f;
             }
         }
         wave_lds_sync();
@@ -231,7 +227,7 @@ state_pass16_kernel(const StatePassArgs a) {
             const int ta = ks * 16 + tr_tok, tb = ta + 4;
 #pragma unroll
             for (int i = 0; i < PBW; ++i) {
-                const int col = pw * (P / 2) + i * 32 + tr_col;
+                const int col = i * 32 + tr_col;
                 const tvec4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
                     (M2_LDS tvec4*)(cX + (ta * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(ta))) * 8 + (col & 7)));
                 const tvec4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(

@@ -78,9 +78,11 @@ __device__ __forceinline__ void async_copy_ldtab(const float* __restrict__ ldtab
 //   row-wise fragments : 16 consecutive rows, one slot each          -> 16 different (row parity, slot) bank groups
 //   transpose reads    : 4 consecutive rows (aligned), 4 slots each   -> the rows' 4-slot groups must differ
 // which a bit permutation of the row index gives (256-byte rows: swap the two low bit pairs; 128-byte rows: bit 0
-// already selects the bank half, bits 1..3 go to slot bits 2, 0, 1).
+// already selects the bank half, bits 1..3 go to slot bits 2, 0, 1; 64-byte rows: four consecutive rows are 256 contiguous
+// bytes, which is what either access covers, so no permutation is needed).
 template <int SPR> __device__ __forceinline__ int tile_swz(int row) {
-    static_assert(SPR == 8 || SPR == 16, "tile rows of 128 or 256 bytes");
+    static_assert(SPR == 4 || SPR == 8 || SPR == 16, "tile rows of 64, 128 or 256 bytes");
+    if (SPR == 4) return 0;
     if (SPR == 16) return ((row & 3) << 2) | ((row >> 2) & 3);
     return (((row >> 1) & 1) << 2) | (((row >> 3) & 1) << 1) | ((row >> 2) & 1);
 }
