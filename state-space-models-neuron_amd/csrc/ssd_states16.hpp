@@ -18,7 +18,8 @@
 //   * x / dy rows are loaded one chunk ahead into registers, scaled per token in fp32, rounded once and written
 //     row-major into one of two LDS buffers (one barrier per chunk); the A-operand fragments (k = token contiguous)
 //     come out of it through LDS transpose reads.
-// The state leaves through a wave-private LDS tile so that each lane stores 16 contiguous bytes of a state row.
+// The state leaves through an LDS tile of the workgroup's whole slab (one per chunk parity), written before the chunk's barrier
+// and read behind it, so that a wave stores whole state rows: its share of the slab is one contiguous piece of memory.
 #pragma once
 #include "ssd_y.hpp"
 
@@ -43,7 +44,7 @@ constexpr int kStatePassSplit = 2;
 template <int N> constexpr int state_pass_threads() { return (N / 32) * 64; }
 template <int P, int N>
 constexpr size_t state_pass_smem() {
-    return (size_t)2 * kQ * (P / 2) * 2 + (size_t)(N / 32) * (P / 2) * (32 + 8) * 2;
+    return (size_t)2 * kQ * (P / 2) * 2 + (size_t)2 * (P / 2) * (N + 8) * 2;
 }
 
 template <typename T, int P, int N, bool REVERSE, bool DLAM = REVERSE>
@@ -57,13 +58,15 @@ state_pass16_kernel(const StatePassArgs a) {
     constexpr int PBW = PH / 32, NBW = 1;              // 32x32 blocks per wave
     constexpr int SPR_X = PH / 8;                      // 16-byte slots per staged x row
     constexpr int NXR = kQ * SPR_X / THREADS;              // x pieces per thread per chunk
-    constexpr int LDO = NW + 8;
-    constexpr int LPR = NW / 8;                   // lanes per row of this wave's state block (8 elements each)
+    constexpr int LDO = N + 8;
+    constexpr int LPR = N / 8;                         // lanes per state row (8 elements each)
     constexpr int RPP = 64 / LPR;                      // rows per store pass
-    constexpr int NSP = (P / 2) / RPP;                 // store passes
+    constexpr int RW = PH / NWAVES;                    // rows a wave stores: the workgroup's slab leaves as whole rows
+    constexpr int NSP = RW / RPP;                      // store passes
+    static_assert(RW % RPP == 0, "whole store passes");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* sX = reinterpret_cast<T*>(smem_raw);                                 // [2][kQ][P / 2], slots swizzled inside each row
-    T* sO = sX + 2 * kQ * PH;                                               // [waves][P / 2][LDO]
+    T* sO = sX + 2 * kQ * PH;                                               // [2][P / 2][LDO]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 31, half = lane >> 5;
@@ -75,7 +78,6 @@ state_pass16_kernel(const StatePassArgs a) {
     const int64_t g = h / (a.nheads / a.ngroups);
     const int64_t bh = b * a.nheads + h;
     const int64_t nc = a.nchunks;
-    T* sOw = sO + wave * (P / 2) * LDO;
     const int tr_tok = 8 * half + ((lane >> 2) & 3);
     const int tr_col = ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
     typedef T tvec4 __attribute__((ext_vector_type(4)));
@@ -128,7 +130,7 @@ state_pass16_kernel(const StatePassArgs a) {
     Frag<T> bf[NBW][8];
     static_assert(REVERSE || !DLAM, "dlam belongs to the reverse pass");
     u32x4 spr[DLAM ? NSP : 1];
-    const uint32_t st_off = (uint32_t)(((pw * (P / 2) + lane / LPR) * N + n0 + (lane % LPR) * 8) * 2);      // pass ps: + ps * RPP * N * 2
+    const uint32_t st_off = (uint32_t)(((pw * PH + wave * RW + lane / LPR) * N + (lane % LPR) * 8) * 2);      // pass ps: + ps * RPP * N * 2
     auto load_same = [&](int64_t c) {
         const char* mp = reinterpret_cast<const char*>(static_cast<const T*>(a.Mt) + ((b * nc + c) * a.ngroups + g) * (int64_t)(N * kQ));
 #pragma unroll
@@ -176,11 +178,9 @@ state_pass16_kernel(const StatePassArgs a) {
             *reinterpret_cast<u32x4*>(cX + (row * SPR_X + (slot ^ tile_swz<SPR_X>(row))) * 8) = o;
         }
         const float dec = __expf(s.lam);
-        __syncthreads();          // the tile is complete; every wave is done with the other buffer
-        // the rows two chunks on (past the end: the last chunk once more, rather than branching around the loads)
-        load_ahead(chunk_of(cc + 2), s);
-
-        // ---- the state entering (forward) / the gradient leaving (reverse) this chunk, through the wave-private tile
+        // the state as it enters this chunk goes into the slab tile of this parity (the other one may still be read by a
+        // wave that is behind: it was filled one barrier ago)
+        T* cO = sO + buf * (PH * LDO);
 #pragma unroll
         for (int i = 0; i < PBW; ++i)
 #pragma unroll
@@ -188,15 +188,19 @@ state_pass16_kernel(const StatePassArgs a) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const uint2 w = {pack2<T>(acc[i][j][4 * q], acc[i][j][4 * q + 1]), pack2<T>(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3])};
-                    *reinterpret_cast<uint2*>(sOw + (i * 32 + r) * LDO + j * 32 + 8 * q + 4 * half) = w;
+                    *reinterpret_cast<uint2*>(cO + (i * 32 + r) * LDO + n0 + j * 32 + 8 * q + 4 * half) = w;
                 }
-        wave_lds_sync();
+        __syncthreads();          // both tiles are complete; every wave is done with the other buffers
+        // the rows two chunks on (past the end: the last chunk once more, rather than branching around the loads)
+        load_ahead(chunk_of(cc + 2), s);
+
+        // ---- the state entering (forward) / the gradient leaving (reverse) this chunk: whole rows of the workgroup's slab
         char* op = reinterpret_cast<char*>(static_cast<T*>(a.prev) + ((b * nc + c) * a.nheads + h) * (int64_t)(P * N));
         float dot = 0.f;
 #pragma unroll
         for (int ps = 0; ps < NSP; ++ps) {
-            const int rl = ps * RPP + lane / LPR, cv = lane % LPR;
-            const u32x4 o = *reinterpret_cast<const u32x4*>(sOw + rl * LDO + cv * 8);
+            const int rl = wave * RW + ps * RPP + lane / LPR, cv = lane % LPR;
+            const u32x4 o = *reinterpret_cast<const u32x4*>(cO + rl * LDO + cv * 8);
             *reinterpret_cast<u32x4*>(op + (st_off + (uint32_t)(ps * RPP * N * 2))) = o;
             if (DLAM) {
 #pragma unroll
@@ -213,7 +217,6 @@ state_pass16_kernel(const StatePassArgs a) {
                     a.dlam[(bh * nc + c) * kDlamParts + slot + kStatePassSplit * NWAVES] = 0.f;
             }
         }
-        wave_lds_sync();
 
         // ---- S = e^{Lam} S + X_scaled^T M  (accumulated as its transpose M^T X_scaled)
 #pragma unroll
