@@ -27,7 +27,7 @@ constexpr int kMaxK = 8;
 #define M2_CONV_TLF 16
 #endif
 #ifndef M2_CONV_TLB
-#define M2_CONV_TLB 64
+#define M2_CONV_TLB 32
 #endif
 #ifndef M2_CONV_UNR
 #define M2_CONV_UNR 4
@@ -36,10 +36,12 @@ constexpr int kMaxK = 8;
 #define M2_CONV_VF 8
 #endif
 #ifndef M2_CONV_VB
-#define M2_CONV_VB 8
+#define M2_CONV_VB 4
 #endif
-// Tokens per thread in the fast path.  The forward is short on loads in flight, so it takes short segments (many
-// threads); the backward carries more per-thread state and recomputes 3 lag tokens per segment, so it takes long ones.
+// Tokens per thread in the fast path, and bytes of channels per thread (VF forward, VB backward; at least two channels).
+// Both directions are short on loads in flight, so they take short segments (many threads).  The backward carries five
+// sums, two 3-token windows and the taps per channel: with two channels per thread it needs 96 registers (five waves per
+// SIMD), with four 160 (three waves), and the narrower form is the faster one although its loads are 4-byte ones.
 constexpr int kTLF = M2_CONV_TLF;
 constexpr int kTLB = M2_CONV_TLB;
 constexpr int kUNR = M2_CONV_UNR;    // tokens whose loads are in flight together
@@ -456,7 +458,10 @@ conv_bwd_dw_generic_kernel(const T* __restrict__ x, const void* __restrict__ w, 
 
 // elements per thread: 16-byte vectors forward, 8-byte vectors backward (the backward carries twice the
 // per-channel state in registers; halving the vector keeps its occupancy up)
-template <typename T> constexpr int conv_vec(bool bwd) { return (int)(bwd ? M2_CONV_VB / sizeof(T) : M2_CONV_VF / sizeof(T)); }
+template <typename T> constexpr int conv_vec(bool bwd) {
+    const int v = (int)((bwd ? M2_CONV_VB : M2_CONV_VF) / sizeof(T));
+    return v < 2 ? 2 : v;
+}
 
 template <typename T, int V>
 bool fast_path_ok(const m2_conv1d_params* p, bool bwd) {
