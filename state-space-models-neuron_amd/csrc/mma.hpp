@@ -84,6 +84,13 @@ template <typename T> __device__ __forceinline__ float unpack_lo(uint32_t w);
 template <typename T> __device__ __forceinline__ float unpack_hi(uint32_t w);
 template <> __device__ __forceinline__ float unpack_lo<bf16_t>(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
 template <> __device__ __forceinline__ float unpack_hi<bf16_t>(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+// c + a.lo * b.lo + a.hi * b.hi for two words of 16-bit pairs in one instruction (v_dot2c_f32_bf16): the products of two
+// 8-bit significands are exact in fp32, so this is the same sum as two FMAs on unpacked values, without the four unpacks
+template <typename T> __device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t b, float c);
+template <> __device__ __forceinline__ float dot2_acc<bf16_t>(uint32_t a, uint32_t b, float c) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2, a), __builtin_bit_cast(bf2, b), c, false);
+}
 template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     typedef T tvec2 __attribute__((ext_vector_type(2)));
     const tvec2 v = {from_f32<T>(lo), from_f32<T>(hi)};

@@ -132,7 +132,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
             const uint4 v = *reinterpret_cast<const uint4*>(cP + (it * 512 + t) * 8);
             const uint32_t uw[4] = {u.x, u.y, u.z, u.w}, vw[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-            for (int q = 0; q < 4; ++q) dot += unpack_lo<T>(uw[q]) * unpack_lo<T>(vw[q]) + unpack_hi<T>(uw[q]) * unpack_hi<T>(vw[q]);
+            for (int q = 0; q < 4; ++q) dot = dot2_acc<T>(uw[q], vw[q], dot);
         }
         dot = warp_sum(dot);
         if (lane == 0) a.dlam[bhc * kDlamParts + wave] = __expf(Lam) * dot;
@@ -294,7 +294,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                         const float y0 = unpack_lo<T>(gw[e]), y1 = unpack_hi<T>(gw[e]);
                         ow[e] = pack2<T>(dtt * d0 + Dh * y0, dtt * d1 + Dh * y1);
                         dir += d0 * x0 + d1 * x1;
-                        dd += y0 * x0 + y1 * x1;
+                        dd = dot2_acc<T>(gw[e], xw[e], dd);
                     }
                     if (tok < valid) *reinterpret_cast<uint4*>(dXp + p0) = uint4{ow[0], ow[1], ow[2], ow[3]};
                 }

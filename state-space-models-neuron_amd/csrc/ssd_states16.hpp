@@ -205,7 +205,7 @@ state_pass16_kernel(const StatePassArgs a) {
             if (DLAM) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
-                    dot += unpack_lo<T>(o[q]) * unpack_lo<T>(spr[ps][q]) + unpack_hi<T>(o[q]) * unpack_hi<T>(spr[ps][q]);
+                    dot = dot2_acc<T>(o[q], spr[ps][q], dot);
             }
         }
         if (DLAM) {
