@@ -272,7 +272,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
             //      4-channel group leaves every lane with whole groups of 8 consecutive channels of its token: 16-byte
             //      reads of x and dy, 16-byte stores of dx, no pass through LDS
             T* dXp = static_cast<T*>(a.dx) + b * a.dx_sb + t0 * a.dx_sl + h * a.dx_sh + (int64_t)tok * a.dx_sl;
-            const float dtt = sd[tok];
+            const float dts = sd[tok] * fin_sc;      // the block's final scale rides on dt here and on the finished row sum below
             float dir = 0.f, dd = 0.f;
 #pragma unroll
             for (int j = 0; j < BN; ++j) {
@@ -289,10 +289,10 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                     uint32_t ow[4];
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const float d0 = fin_sc * g8[2 * e], d1 = fin_sc * g8[2 * e + 1];
+                        const float d0 = g8[2 * e], d1 = g8[2 * e + 1];
                         const float x0 = unpack_lo<T>(xw[e]), x1 = unpack_hi<T>(xw[e]);
                         const float y0 = unpack_lo<T>(gw[e]), y1 = unpack_hi<T>(gw[e]);
-                        ow[e] = pack2<T>(dtt * d0 + Dh * y0, dtt * d1 + Dh * y1);
+                        ow[e] = pack2<T>(dts * d0 + Dh * y0, dts * d1 + Dh * y1);
                         dir += d0 * x0 + d1 * x1;
                         dd = dot2_acc<T>(gw[e], xw[e], dd);
                     }
@@ -300,7 +300,7 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                 }
             }
             dir = lane_xor_add<32>(dir);
-            if (half == 0) a.dirp[bhc * kQ + tok] = dir;
+            if (half == 0) a.dirp[bhc * kQ + tok] = dir * fin_sc;
             float dD_loc = warp_sum(tok < valid ? dd : 0.f);
             if (lane == 0) { a.dDp8[bhc * 8 + wave] = dD_loc; a.dDp8[bhc * 8 + wave + 4] = 0.f; }
         }
