@@ -174,8 +174,10 @@ rmsnorm_gated_kernel(const NormArgs a) {
     // the raw vectors of the next row are loaded before this row is reduced (the row after the last: the last once more)
     constexpr int RSTEP = WPG == 4 ? 1 : 4;
     const bool gated = a.z != nullptr;
-    uint4 rx[NV], rz[NV], rg[BWD ? NV : 1];
-    auto load_row = [&](int64_t r) {
+    // the forward keeps two register sets and loads a row a whole iteration before it is used (the backward has no
+    // registers left for that: it loads the next row behind the first pass over the current one)
+    uint4 rxa[NV], rza[NV], rxb[BWD ? 1 : NV], rzb[BWD ? 1 : NV], rg[BWD ? NV : 1];
+    auto load_row = [&](int64_t r, uint4 (&rx)[NV], uint4 (&rz)[NV]) {
         const int64_t rr = r < r1 ? r : r1 - 1;
         const T* xr = static_cast<const T*>(a.x) + rr * a.x_sr + c0;
         const T* zr = gated ? static_cast<const T*>(a.z) + rr * a.z_sr + c0 : xr;
@@ -190,8 +192,8 @@ rmsnorm_gated_kernel(const NormArgs a) {
         }
     };
     const int64_t rfirst = r0 + (WPG == 4 ? 0 : wave);
-    if (rfirst < r1) load_row(rfirst);
-    for (int64_t r = rfirst; r < r1; r += RSTEP) {
+    if (rfirst < r1) load_row(rfirst, rxa, rza);
+    auto do_row = [&](int64_t r, uint4 (&rx)[NV], uint4 (&rz)[NV]) {
         const bool zr = gated;
         float h[NV][V], xs[BWD ? NV : 1][V], zs[BWD ? NV : 1][V], gs[BWD ? NV : 1][V];
         float ss = 0.f, dot = 0.f;
@@ -214,7 +216,7 @@ rmsnorm_gated_kernel(const NormArgs a) {
                 }
             }
         }
-        load_row(r + RSTEP);
+        if (BWD) load_row(r + RSTEP, rx, rz);
         group_sum2<WPG>(ss, dot, red, slot);
         slot ^= 1;
         const float var = ss * inv_n + a.eps;
@@ -254,6 +256,19 @@ rmsnorm_gated_kernel(const NormArgs a) {
                 }
                 store_vec<T>(static_cast<T*>(a.dx) + r * a.dx_sr + c0 + (int64_t)vi * V, ox);
                 if (zr && a.dz) store_vec<T>(static_cast<T*>(a.dz) + r * a.dz_sr + c0 + (int64_t)vi * V, oz);
+            }
+        }
+    };
+    if constexpr (BWD) {
+        for (int64_t r = rfirst; r < r1; r += RSTEP) do_row(r, rxa, rza);
+    } else {
+        // rows in pairs, one per register set; a row's loads are issued before the row in front of it is processed
+        for (int64_t r = rfirst; r < r1; r += 2 * RSTEP) {
+            load_row(r + RSTEP, rxb, rzb);
+            do_row(r, rxa, rza);
+            if (r + RSTEP < r1) {      // uniform over the workgroup when it shares its rows (WPG == 4)
+                load_row(r + 2 * RSTEP, rxa, rza);
+                do_row(r + RSTEP, rxb, rzb);
             }
         }
     }
