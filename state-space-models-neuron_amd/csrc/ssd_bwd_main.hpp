@@ -94,28 +94,34 @@ ssd_bwd16_kernel(const Bwd16Args a) {
         const T* Sp = static_cast<const T*>(a.dS) + tile;
         const T* Pp = static_cast<const T*>(a.Sprev) + tile;
         const uint32_t dst = lds_T + (uint32_t)(buf * TILES * 2);
-        // the per-lane source offsets are recomputed for every head on purpose (a handful of integer instructions):
-        // kept in registers across the head loop they are the first thing the register allocator spills, and a
-        // spill reload in the middle of this sequence waits for all copies issued so far
-        int ln = lane;
+        // the per-lane source offsets are rebuilt for every head on purpose: kept in registers across the head loop they are
+        // the first thing the register allocator spills, and a spill reload in the middle of this sequence waits for all
+        // copies issued so far.  Rebuilding is cheap because the swizzle splits into a lane part, formed once here, and a
+        // chunk part that is wave-uniform (copy_lane_slot / copy_chunk_swz); the row products are 24-bit multiply-adds.
+        uint32_t ln = (uint32_t)lane;
         asm volatile("" : "+v"(ln));
+        constexpr int RPC_S = 64 / SPR_S, RPC_X = 64 / SPR_X;       // tile rows per 64-slot chunk
+        const uint32_t sS = copy_lane_slot<SPR_S>(ln), sX = copy_lane_slot<SPR_X>(ln);
+        const uint32_t lrS = ln / (uint32_t)SPR_S, lrX = ln / (uint32_t)SPR_X;
+        const uint32_t baseS = lrS * (uint32_t)(N * 2) + (sS << 4);                 // row and slot fields do not overlap
 #pragma unroll
         for (int it = 0; it < NS; ++it) {
-            const int s = (int)(wave_u * NS + it) * 64 + ln;
-            const int row = s / SPR_S, cs = (s % SPR_S) ^ tile_swz<SPR_S>(row);
-            const uint32_t off = (uint32_t)(row * N + cs * 8) * 2u;
-            async_copy16(Sp, off, dst + (wave_u * NS + it) * 1024u);
-            async_copy16(Pp, off, dst + (uint32_t)(P * N * 2) + (wave_u * NS + it) * 1024u);
+            const uint32_t ch = wave_u * NS + it;
+            const uint32_t off = ch * (uint32_t)(RPC_S * N * 2) + (baseS ^ (copy_chunk_swz<SPR_S>(ch) << 4));
+            async_copy16(Sp, off, dst + ch * 1024u);
+            async_copy16(Pp, off, dst + (uint32_t)(P * N * 2) + ch * 1024u);
         }
         const T* Yp = static_cast<const T*>(a.dy) + b * a.dy_sb + t0 * a.dy_sl + h * a.dy_sh;
         const T* Xp = static_cast<const T*>(a.x) + b * a.x_sb + t0 * a.x_sl + h * a.x_sh;
+        const uint32_t ypitch = uniform((uint32_t)a.dy_sl * 2u), xpitch = uniform((uint32_t)a.x_sl * 2u), last = (uint32_t)(valid - 1);
 #pragma unroll
         for (int it = 0; it < NX; ++it) {
-            const int s = (int)(wave_u * NX + it) * 64 + ln;
-            const int row = s / SPR_X, cs = (s % SPR_X) ^ tile_swz<SPR_X>(row);
-            const int grow = row < valid ? row : valid - 1;       // rows past the end: finite stand-ins, masked by zero scales
-            async_copy16(Yp, (uint32_t)(grow * a.dy_sl + cs * 8) * 2u, dst + (uint32_t)(2 * P * N * 2) + (wave_u * NX + it) * 1024u);
-            async_copy16(Xp, (uint32_t)(grow * a.x_sl + cs * 8) * 2u, dst + (uint32_t)((2 * P * N + kQ * P) * 2) + (wave_u * NX + it) * 1024u);
+            const uint32_t ch = wave_u * NX + it;
+            const uint32_t row = ch * RPC_X + lrX;
+            const uint32_t grow = row < last ? row : last;       // rows past the end: finite stand-ins, masked by zero scales
+            const uint32_t cs16 = (sX ^ copy_chunk_swz<SPR_X>(ch)) << 4;
+            async_copy16(Yp, __umul24(grow, ypitch) + cs16, dst + (uint32_t)(2 * P * N * 2) + ch * 1024u);
+            async_copy16(Xp, __umul24(grow, xpitch) + cs16, dst + (uint32_t)((2 * P * N + kQ * P) * 2) + ch * 1024u);
         }
         async_copy_ldtab(a.ldtab, (b * a.nheads + h) * a.nchunks + c, lds_LD + (uint32_t)(buf * 2 * kQ * 4));
     };

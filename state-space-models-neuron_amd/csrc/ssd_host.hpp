@@ -137,6 +137,15 @@ inline int ssd_check(const m2_ssd_params* p, const char* who) {
                p->C_stride_b % V == 0 && p->C_stride_l % V == 0 && p->C_stride_g % V == 0,
                M2_ERR_ALIGN, "%s: x/B/C strides must be multiples of %d elements (16 bytes)", who, V);
     M2_REQUIRE(aligned16(p->x) && aligned16(p->B) && aligned16(p->C), M2_ERR_ALIGN, "%s: x/B/C must be 16-byte aligned", who);
+    {
+        // the kernels address the rows of a chunk with 32-bit byte offsets formed by 24-bit multiplies
+        const int64_t lim = (int64_t)1 << 21;
+        auto ok = [&](int64_t s) { return s >= 0 && s < lim; };
+        M2_REQUIRE(ok(p->x_stride_l) && ok(p->B_stride_l) && ok(p->C_stride_l) && ok(p->dt_stride_l) && (!p->y || ok(p->y_stride_l)),
+                   M2_ERR_SHAPE, "%s: token strides must lie in [0, 2^21) elements", who);
+        M2_REQUIRE(!p->dy || (ok(p->dy_stride_l) && ok(p->dx_stride_l) && ok(p->dB_stride_l) && ok(p->dC_stride_l) && ok(p->ddt_stride_l)),
+                   M2_ERR_SHAPE, "%s: token strides of the gradients must lie in [0, 2^21) elements", who);
+    }
     M2_REQUIRE(aligned16(p->chunk_states), M2_ERR_ALIGN, "%s: chunk_states must be 16-byte aligned", who);
     return M2_OK;
 }

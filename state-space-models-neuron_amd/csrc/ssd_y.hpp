@@ -87,6 +87,19 @@ template <int SPR> __device__ __forceinline__ int tile_swz(int row) {
     return (((row >> 1) & 1) << 2) | (((row >> 3) & 1) << 1) | ((row >> 2) & 1);
 }
 
+// The same swizzle split for the direct-to-LDS copies: lane `ln` of 64-slot chunk `ch` of a tile fills slot ln % SPR of row
+// ch * (64 / SPR) + ln / SPR, and tile_swz of that row is the XOR of a part that depends on the lane alone and a part that
+// depends on the (wave-uniform) chunk alone, so the per-lane work of a copy is one XOR on a value computed once per head.
+template <int SPR> __device__ __forceinline__ uint32_t copy_lane_slot(uint32_t ln) {      // (ln % SPR) ^ lane part of tile_swz
+    static_assert(SPR == 8 || SPR == 16, "tile rows of 128 or 256 bytes");
+    if (SPR == 16) return (ln & 15u) ^ ((ln >> 4) << 2);
+    const uint32_t lr = ln >> 3;
+    return (ln & 7u) ^ ((((lr >> 1) & 1u) << 2) | ((lr >> 2) & 1u));
+}
+template <int SPR> __device__ __forceinline__ uint32_t copy_chunk_swz(uint32_t ch) {      // chunk part of tile_swz
+    return SPR == 16 ? (ch & 3u) : ((ch & 1u) << 1);
+}
+
 template <int P, int N>
 constexpr size_t y16_smem() {
     return (size_t)2 * ((P * N + kQ * P) * 2 + 2 * kQ * sizeof(float)) + (size_t)4 * (kQ + 32) * sizeof(float);
