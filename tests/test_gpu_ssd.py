@@ -114,6 +114,29 @@ def test_ssd_rejects_unsupported():
         mamba2_kernel(d["dt"], d["A"], d["X"], d["B"], d["C"], d["D"])
 
 
+def test_ssd_rejects_token_strides_beyond_the_offset_arithmetic():
+    """The kernels form row offsets inside a chunk with 24-bit multiplies and 32-bit sums: a token stride of 2^21 elements or
+    more is refused by the library before anything is launched (checked straight through the C ABI: no tensor has such a stride)."""
+    from mamba2 import _lib
+    from mamba2._lib import SsdParams, ptr
+    from mamba2.mamba2_kernel import _fill_common, _strides3
+    d = _dev(make_ssd_inputs(1, 128, 2, 64, 64, 1, seed=0, dtype=torch.bfloat16))
+    lib = _lib.load()
+    Y = torch.empty_like(d["X"])
+    p = SsdParams()
+    _fill_common(p, d["dt"], d["A"].float(), d["X"], d["B"], d["C"], None)
+    p.y = ptr(Y)
+    p.y_stride_b, p.y_stride_l, p.y_stride_h = _strides3(Y)
+    ws = torch.empty(lib.m2_ssd_fwd_workspace_bytes(p), dtype=torch.uint8, device=DEV)
+    p.workspace, p.workspace_bytes = ptr(ws), ws.numel()
+    p.x_stride_l = 1 << 21
+    rc = lib.m2_ssd_fwd(p, _lib.stream_ptr(torch.device(DEV)))
+    assert rc == -1 and b"token strides" in lib.m2_last_error()      # M2_ERR_SHAPE
+    p.x_stride_l = d["X"].stride(1)
+    assert lib.m2_ssd_fwd(p, _lib.stream_ptr(torch.device(DEV))) == 0
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("b,l,h,p,n,g", CASES)
 def test_ssd_backward(dtype, b, l, h, p, n, g):
