@@ -28,6 +28,9 @@ CASES = [
     (1, 200, 2, 128, 64, 1),     # ragged length, p = 128
     (2, 128, 4, 128, 128, 4),
     (1, 77, 2, 64, 128, 1),      # shorter than one chunk
+    (1, 640, 2, 128, 128, 2),    # p = 128 over an odd number of chunks (the state pass peels one off)
+    (1, 512, 4, 128, 64, 1),     # p = 128, n = 64 over an even number
+    (2, 896, 4, 64, 64, 2),      # n = 64: two-wave state pass, seven chunks
 ]
 
 
