@@ -64,6 +64,16 @@ __device__ __forceinline__ void async_copy16(const void* gbase, uint32_t voff, u
 __device__ __forceinline__ uint32_t lds_addr_of(const void* p) { return (uint32_t)(uintptr_t)(M2_LDS const void*)p; }
 __device__ __forceinline__ uint32_t uniform(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 
+// One float at a wave-uniform address through the scalar cache.  The head loops use it for per-head parameters: an ordinary
+// load there is a vector-memory operation that the compiler counts on its own, without knowing of the direct-to-LDS copies
+// around it, so the wait it puts in front of the value's first use is a vmcnt(0) -- a wait for the NEXT head's tiles in
+// front of this head's arithmetic.
+__device__ __forceinline__ float load_uniform_f32(const float* p) {
+    float v;
+    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(p) : "memory");
+    return v;
+}
+
 // The [ l | dt ] table of one (batch, head, chunk): 2 kQ floats = 64 lanes x 16 bytes, one wave-wide copy.  Every
 // wave of the workgroup issues it (same source, same destination, same data), so each wave may read the table as
 // soon as ITS OWN copies have landed, and all waves issue the same number of vector-memory operations per head.
@@ -182,9 +192,12 @@ ssd_y16_kernel(const DiagArgs a) {
     for (int64_t hh = 0; hh < a.hps; ++hh) {
         const int64_t h = h_first + hh;
         const int buf = (int)(hh & 1);
-        const float Dh = a.D ? a.D[h] : 0.f;
+        const float Dh = a.D ? load_uniform_f32(a.D + h) : 0.f;
 
-        wait_vmem_all();          // this wave's share of the tiles of head hh, and the whole [ l | dt ] table, have landed
+        // this wave's share of the tiles of head hh, and the whole [ l | dt ] table, have landed.  The y stores of the head
+        // before were issued behind these copies and vector-memory operations retire in issue order, so in a full chunk
+        // (every lane stores, 2 BN instructions per head) they may stay in flight across the wait
+        if (hh > 0 && valid == kQ) wait_vmem_keep<2 * BN>(1); else wait_vmem_all();
         // ---- wave-private decay tables from the shared [ l | dt ] table
         const float* sl = sLD + buf * 2 * kQ;
         const float* sd = sl + kQ;
