@@ -225,6 +225,9 @@ state_pass16_kernel(const StatePassArgs a) {
             for (int j = 0; j < NBW; ++j)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] *= dec;
+        // all A-operand fragments of the chunk are read from LDS first: the eight products form one dependent chain, and a
+        // read issued next to its product would put an LDS round trip between any two of them
+        Frag<T> af[PBW][8];
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             const int ta = ks * 16 + tr_tok, tb = ta + 4;
@@ -235,13 +238,17 @@ state_pass16_kernel(const StatePassArgs a) {
                     (M2_LDS tvec4*)(cX + (ta * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(ta))) * 8 + (col & 7)));
                 const tvec4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
                     (M2_LDS tvec4*)(cX + (tb * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(tb))) * 8 + (col & 7)));
-                Frag<T> af;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { af.v[e] = lo[e]; af.v[4 + e] = hi[e]; }
-#pragma unroll
-                for (int j = 0; j < NBW; ++j) mma_frag(acc[i][j], bf[j][ks], af);
+                for (int e = 0; e < 4; ++e) { af[i][ks].v[e] = lo[e]; af[i][ks].v[4 + e] = hi[e]; }
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+            for (int i = 0; i < PBW; ++i)
+#pragma unroll
+                for (int j = 0; j < NBW; ++j) mma_frag(acc[i][j], bf[j][ks], af[i][ks]);
     };
 
     // Chunks are taken two per loop iteration (one per register set); an odd first chunk is peeled off in front so that
