@@ -28,6 +28,7 @@ def lib():
 
 
 PARITY_LOG = []
+PARITY_LOG_DIR = os.environ.get("M2_PARITY_LOG_DIR") or os.path.join(ROOT, "gpurun_out")      # results folder of a GPU run
 
 
 def bf16_floor(ref):
@@ -48,8 +49,8 @@ def raw_rms_err(got, ref):
 def rel_rms_err(got, ref, name=None, extra_floor=0.0, bf16_operands=False):
     """bf16 acceptance metric (bar 2e-2): RAW max |got - ref| / RMS(ref), minus a floor.
 
-    The raw figure is what the bar is stated on and what is recorded (``PARITY_LOG``, written to
-    ``gpurun_out/parity_raw.jsonl`` at the end of the session, one line per comparison: test, tensor, raw, floor).
+    The raw figure is what the bar is stated on and what is recorded (``PARITY_LOG``, written to ``parity_raw.jsonl``
+    in the results folder ``PARITY_LOG_DIR`` at the end of the session, one line per comparison: test, tensor, raw, floor).
     For a result STORED in bfloat16 the exact value itself cannot be represented better than half an ulp (2^-9
     relative), which for heavy-tailed tensors (|ref| > 10 RMS) alone exceeds 2e-2 RMS: floor = max |bf16(ref) - ref|
     / RMS(ref), computed here from the same reference.  ``assert rel_rms_err(got, ref) < 2e-2`` therefore reads
@@ -77,7 +78,7 @@ def pytest_sessionfinish(session, exitstatus):
     if not PARITY_LOG:
         return
     import json
-    out = os.path.join(ROOT, "gpurun_out")
+    out = PARITY_LOG_DIR
     os.makedirs(out, exist_ok=True)
     with open(os.path.join(out, "parity_raw.jsonl"), "w") as f:
         for rec in PARITY_LOG:
