@@ -15,7 +15,7 @@
 //   * M (B or C of the group) comes from the transposed tiles that prep_kernel wrote in MFMA operand order: a wave's
 //     B-operand fragment is one contiguous KiB of global memory, loaded straight into registers at the top of the
 //     chunk's iteration (the tile is shared by all heads of the group and stays in L2);
-//   * x / dy rows are loaded one chunk ahead into registers, scaled per token in fp32, rounded once and written
+//   * x / dy rows are loaded two chunks ahead into registers, scaled per token in fp32, rounded once and written
 //     row-major into one of two LDS buffers (one barrier per chunk); the A-operand fragments (k = token contiguous)
 //     come out of it through LDS transpose reads.
 // The state leaves through an LDS tile of the workgroup's whole slab (one per chunk parity), written before the chunk's barrier
