@@ -348,6 +348,10 @@ ssd_bwd16_kernel(const Bwd16Args a) {
             const int r = ln & 31, half = ln >> 5, tok = row0 + r;
             const int tr_row = (ln >> 2) & 3, tr_col = ((ln >> 4) & 1) * 16 + 4 * (ln & 3);
             tiles_dot(buf, (b * a.nheads + h) * a.nchunks + c, sl[kQ - 1]);
+            // lane parts of the transpose-read addresses into a [P][N] state tile (byte offsets; see rows_times_state)
+            const uint32_t c3 = (uint32_t)(tr_col >> 3);
+            const uint32_t LA = (uint32_t)(8 * half + tr_row) * 256u + ((c3 ^ (uint32_t)(2 * half)) << 4) + (uint32_t)(tr_col & 7) * 2u;
+            const uint32_t LB = (LA ^ 16u) + 1024u, trs = (uint32_t)tr_row << 6;
             // row scales of this lane's token: dt_j e^{Lam - l_j} (dB side) and e^{l_i} (dC side and dl_c; 0 past the end)
             const float lr = sl[tok];
             const float ws_b = sd[tok] * __expf(sl[kQ - 1] - lr);
@@ -362,17 +366,29 @@ ssd_bwd16_kernel(const Bwd16Args a) {
                 Frag<T> af[KSP];
 #pragma unroll
                 for (int ks = 0; ks < KSP; ++ks) af[ks] = load_frag(Rows + (tok * SPR_X + ((ks * 2 + half) ^ tile_swz<SPR_X>(tok))) * 8);
+                const uint32_t sbase = lds_addr_of(St);
 #pragma unroll
                 for (int jn = 0; jn < NBN; ++jn) {
                     floatx16 t = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                     const int col = jn * 32 + tr_col;
+                    // 256-byte state rows: tile_swz of the rows this lane addresses (ks 16 + 8 half + tr_row, and 4 further) does
+                    // not depend on ks, and jn enters the slot only through an XOR with tr_row, so the 16 addresses of a
+                    // column block are two lane values plus compile-time offsets
+                    const uint32_t xj = ((uint32_t)jn << 6) ^ trs;
+                    const uint32_t aA = sbase + LA + xj, aB = sbase + LB + xj;
 #pragma unroll
                     for (int ks = 0; ks < KSP; ++ks) {
                         const int pa = ks * 16 + 8 * half + tr_row, pb = pa + 4;
-                        const tvec4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-                            (M2_LDS tvec4*)(St + (pa * SPR_S + ((col >> 3) ^ tile_swz<SPR_S>(pa))) * 8 + (col & 7)));
-                        const tvec4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-                            (M2_LDS tvec4*)(St + (pb * SPR_S + ((col >> 3) ^ tile_swz<SPR_S>(pb))) * 8 + (col & 7)));
+                        tvec4 lo, hi;
+                        if constexpr (SPR_S == 16) {
+                            lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((M2_LDS tvec4*)(uintptr_t)(aA + (uint32_t)(ks * 16 * 256)));
+                            hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((M2_LDS tvec4*)(uintptr_t)(aB + (uint32_t)(ks * 16 * 256)));
+                        } else {
+                            lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                                (M2_LDS tvec4*)(St + (pa * SPR_S + ((col >> 3) ^ tile_swz<SPR_S>(pa))) * 8 + (col & 7)));
+                            hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                                (M2_LDS tvec4*)(St + (pb * SPR_S + ((col >> 3) ^ tile_swz<SPR_S>(pb))) * 8 + (col & 7)));
+                        }
                         Frag<T> bf;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) { bf.v[e] = lo[e]; bf.v[4 + e] = hi[e]; }
