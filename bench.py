@@ -444,8 +444,8 @@ def cpu_baseline_decode():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all", choices=["all", "ssd", "conv", "glue", "core", "decode", "model", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--exclude", default="", help="comma-separated workloads to leave out of --workload all (for per-kernel profiles)")
