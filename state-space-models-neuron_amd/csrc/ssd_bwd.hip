@@ -431,6 +431,121 @@ bc_final_body(const float* __restrict__ dGp, const float* __restrict__ dCp, cons
         }
 }
 
+// Group-level finish for 16-bit operands, both sides in one workgroup of 8 waves, so that the head-summed dG is read once:
+//   waves 0-3 (row block w):      dC[i][n] = sum_{j<=i} dG[i][j] B[j][n] + dCoff[i][n]
+//   waves 4-7 (row block w - 4):  dB[j][n] = sum_{i>=j} dG[i][j] C[i][n] + dBoff[j][n]
+// (wave w and wave w + 4 share a SIMD: 2w + 2 and 8 - 2w k blocks, ten on every SIMD).  dG is split into hi + lo
+// operand-type tiles in LDS (row-major, 16-byte slots swizzled as everywhere), so the contractions see it at ~2^-17
+// relative: the dC side reads its fragments row-wise, the dB side, which needs dG^T, through LDS transpose reads.  B^T / C^T
+// fragments come straight from the operand-order tiles (one contiguous KiB per fragment), the MFMAs are issued with swapped
+// operands, so a lane owns one token: the accumulators start from 16-byte loads of the summed state parts and leave as
+// 16-byte stores after one lane-pair swap per 4-column group.  One barrier, no pass of the results through LDS.
+// With few (batch, chunk, group) triples the launch is latency-bound and more, shorter workgroups win: BOTH = false runs
+// one side per workgroup (`side_b`), wave w and w + 4 taking the two halves of the state columns of row block w & 3, with
+// all B^T / C^T fragments requested before the barrier.
+template <typename T, int N, bool BOTH>
+__device__ __forceinline__ void
+bc_final16_body(const float* __restrict__ dGs, const float* __restrict__ dCs, const float* __restrict__ dBs,
+                const T* __restrict__ Bt, const T* __restrict__ Ct, T* __restrict__ dB, T* __restrict__ dC,
+                int64_t seqlen, int64_t ngroups, int64_t nchunks,
+                int64_t dBsb, int64_t dBsl, int64_t dBsg, int64_t dCsb, int64_t dCsl, int64_t dCsg, int64_t c, int64_t g, int64_t b,
+                const bool wg_side_b) {
+    static_assert(sizeof(T) == 2, "16-bit operands only");
+    constexpr int NBN = BOTH ? N / 32 : N / 64, SPR = kQ / 8;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* sH = reinterpret_cast<T*>(smem_raw);      // [kQ][kQ] hi part of dG
+    T* sL = sH + kQ * kQ;                        // [kQ][kQ] lo part
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 31, half = lane >> 5;
+    const int64_t t0 = c * kQ;
+    const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
+    const int64_t grp = (b * nchunks + c) * ngroups + g;
+    {
+        const float* gp = dGs + grp * (int64_t)(kQ * kQ);
+#pragma unroll
+        for (int it = 0; it < kQ * kQ / 4 / 512; ++it) {
+            const int e = it * 512 + tid, i = e / (kQ / 4), j4 = (e % (kQ / 4)) * 4;
+            floatx4 v = floatx4{0.f, 0.f, 0.f, 0.f};
+            if ((j4 >> 5) <= (i >> 5)) v = *reinterpret_cast<const floatx4*>(gp + i * kQ + j4);      // blocks above the diagonal are never written
+            const T h0 = from_f32<T>(v[0]), h1 = from_f32<T>(v[1]), h2 = from_f32<T>(v[2]), h3 = from_f32<T>(v[3]);
+            const uint2 hw = {pack2<T>(to_f32(h0), to_f32(h1)), pack2<T>(to_f32(h2), to_f32(h3))};
+            const uint2 lw = {pack2<T>(v[0] - to_f32(h0), v[1] - to_f32(h1)), pack2<T>(v[2] - to_f32(h2), v[3] - to_f32(h3))};
+            const int at = (i * SPR + ((j4 >> 3) ^ tile_swz<SPR>(i))) * 8 + (j4 & 7);
+            *reinterpret_cast<uint2*>(sH + at) = hw;
+            *reinterpret_cast<uint2*>(sL + at) = lw;
+        }
+    }
+    const bool side_b = BOTH ? wave >= 4 : wg_side_b;
+    const int rb = wave & 3, tok = rb * 32 + r;
+    const int n0 = BOTH ? 0 : (wave >> 2) * (N / 2);      // first state column of this wave
+    floatx16 acc[NBN];
+    {
+        const float* op = (side_b ? dBs : dCs) + grp * (int64_t)(kQ * N) + (int64_t)tok * N + n0;
+#pragma unroll
+        for (int nb = 0; nb < NBN; ++nb)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const floatx4 v = *reinterpret_cast<const floatx4*>(op + nb * 32 + 8 * q + 4 * half);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[nb][4 * q + e] = v[e];
+            }
+    }
+    const char* tile = reinterpret_cast<const char*>((side_b ? Ct : Bt) + grp * (int64_t)(N * kQ)) + (n0 / 32) * (8 * 1024);
+    const int ks0 = side_b ? 2 * rb : 0, ks1 = side_b ? 8 : 2 * rb + 2;      // 16-wide k blocks of this wave
+    Frag<T> xpre[BOTH ? 1 : 8][NBN];
+    if constexpr (!BOTH) {
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks)
+            if (ks >= ks0 && ks < ks1) {
+#pragma unroll
+                for (int nb = 0; nb < NBN; ++nb)
+                    xpre[ks][nb].v = *reinterpret_cast<const bf16x8*>(tile + ((uint32_t)lane * 16u + (uint32_t)((nb * 8 + ks) * 1024)));
+            }
+    }
+    __syncthreads();
+    const int tr_tok = 8 * half + ((lane >> 2) & 3), tr_col = rb * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+    typedef T tvec4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+        if (ks < ks0 || ks >= ks1) continue;      // wave-uniform
+        Frag<T> yh, yl;
+        if (!side_b) {
+            const int at = (tok * SPR + ((ks * 2 + half) ^ tile_swz<SPR>(tok))) * 8;
+            yh = load_frag(sH + at);
+            yl = load_frag(sL + at);
+        } else {
+            const int ta = ks * 16 + tr_tok, tb = ta + 4;
+            const int aa = (ta * SPR + ((tr_col >> 3) ^ tile_swz<SPR>(ta))) * 8 + (tr_col & 7);
+            const int ab = (tb * SPR + ((tr_col >> 3) ^ tile_swz<SPR>(tb))) * 8 + (tr_col & 7);
+            const tvec4 h0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((M2_LDS tvec4*)(sH + aa));
+            const tvec4 h1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((M2_LDS tvec4*)(sH + ab));
+            const tvec4 l0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((M2_LDS tvec4*)(sL + aa));
+            const tvec4 l1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((M2_LDS tvec4*)(sL + ab));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { yh.v[e] = h0[e]; yh.v[4 + e] = h1[e]; yl.v[e] = l0[e]; yl.v[4 + e] = l1[e]; }
+        }
+#pragma unroll
+        for (int nb = 0; nb < NBN; ++nb) {
+            Frag<T> xf;      // see mt_offset
+            if constexpr (BOTH) xf.v = *reinterpret_cast<const bf16x8*>(tile + ((uint32_t)lane * 16u + (uint32_t)((nb * 8 + ks) * 1024)));
+            else xf = xpre[ks][nb];
+            mma_frag(acc[nb], xf, yh);
+            mma_frag(acc[nb], xf, yl);
+        }
+    }
+    T* out = (side_b ? dB + b * dBsb + t0 * dBsl + g * dBsg : dC + b * dCsb + t0 * dCsl + g * dCsg) + (int64_t)tok * (side_b ? dBsl : dCsl) + n0;
+#pragma unroll
+    for (int nb = 0; nb < NBN; ++nb)
+#pragma unroll
+        for (int qp = 0; qp < 2; ++qp) {
+            float g8[8];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pair_swap(acc[nb][8 * qp + e], acc[nb][8 * qp + 4 + e], g8[e], g8[4 + e]);
+            const uint4 o = {pack2<T>(g8[0], g8[1]), pack2<T>(g8[2], g8[3]), pack2<T>(g8[4], g8[5]), pack2<T>(g8[6], g8[7])};
+            if (tok < valid) *reinterpret_cast<uint4*>(out + nb * 32 + 8 * (2 * qp + half)) = o;
+        }
+}
+
 // dA[h] = sum_{b,c} dAp[b][h][c], dD likewise (fixed order, no atomics).  One workgroup of 512 threads per head.
 __device__ __forceinline__ void ad_reduce_body(const float* __restrict__ dAp, const float* __restrict__ dDp, const float* __restrict__ dbp,
                                                float* __restrict__ dA, float* __restrict__ dD, float* __restrict__ dbias,
@@ -457,27 +572,35 @@ __device__ __forceinline__ void ad_reduce_body(const float* __restrict__ dAp, co
     }
 }
 
-// The group-level finish and the per-head reductions in one launch: the first 2 n_bc workgroups run bc_final_body for
-// (side, chunk, group, batch) = the index split in that order (side 0: dC, side 1: dB -- two independent products,
-// so two workgroups), the others ad_reduce_body for one head each.
+// The group-level finish and the per-head reductions in one launch: the first workgroups run the group finish for
+// ([side,] chunk, group, batch) = the index split in that order (fp32 operands: side 0 dC, side 1 dB, one workgroup each;
+// 16-bit operands with BOTH: both sides in one workgroup), the others ad_reduce_body for one head each.
+constexpr int64_t kTail2BothFrom = 256;      // (batch, chunk, group) triples from which a workgroup takes both sides: one per CU
 struct Tail2Args {
     const float* dGp; const float* dCp; const float* dBp; const void* Bt; const void* Ct; void* dB; void* dC;
     int64_t dBsb, dBsl, dBsg, dCsb, dCsl, dCsg;
     const float* dAp; const float* dDp; const float* dbp; float* dA; float* dD; float* dbias;
     int64_t seqlen, ngroups, nchunks, batch, nheads, n_bc;
 };
-template <typename T, int N>
+template <typename T, int N, bool BOTH>
 __global__ void __launch_bounds__(512)
 tail2_kernel(const Tail2Args a) {
     const int64_t blk = blockIdx.x;
-    if (blk < 2 * a.n_bc) {
-        const int64_t q = blk >> 1;
+    constexpr int SIDES = BOTH ? 1 : 2;
+    static_assert(!BOTH || sizeof(T) == 2, "both sides in one workgroup: 16-bit operands only");
+    if (blk < SIDES * a.n_bc) {
+        const int64_t q = blk / SIDES;
         const int64_t c = q % a.nchunks, g = (q / a.nchunks) % a.ngroups, b = q / (a.nchunks * a.ngroups);
-        bc_final_body<T, N>(a.dGp, a.dCp, a.dBp, static_cast<const T*>(a.Bt), static_cast<const T*>(a.Ct), static_cast<T*>(a.dB),
-                            static_cast<T*>(a.dC), a.seqlen, a.ngroups, a.nchunks, a.dBsb, a.dBsl, a.dBsg, a.dCsb, a.dCsl, a.dCsg, c, g, b,
-                            (blk & 1) != 0);
+        if constexpr (sizeof(T) == 2)
+            bc_final16_body<T, N, BOTH>(a.dGp, a.dCp, a.dBp, static_cast<const T*>(a.Bt), static_cast<const T*>(a.Ct), static_cast<T*>(a.dB),
+                                        static_cast<T*>(a.dC), a.seqlen, a.ngroups, a.nchunks, a.dBsb, a.dBsl, a.dBsg, a.dCsb, a.dCsl, a.dCsg, c, g,
+                                        b, (blk & 1) != 0);
+        else
+            bc_final_body<T, N>(a.dGp, a.dCp, a.dBp, static_cast<const T*>(a.Bt), static_cast<const T*>(a.Ct), static_cast<T*>(a.dB),
+                                static_cast<T*>(a.dC), a.seqlen, a.ngroups, a.nchunks, a.dBsb, a.dBsl, a.dBsg, a.dCsb, a.dCsl, a.dCsg, c, g, b,
+                                (blk & 1) != 0);
     } else {
-        ad_reduce_body(a.dAp, a.dDp, a.dbp, a.dA, a.dD, a.dbias, a.batch, a.nheads, a.nchunks, blk - 2 * a.n_bc);
+        ad_reduce_body(a.dAp, a.dDp, a.dbp, a.dA, a.dD, a.dbias, a.batch, a.nheads, a.nchunks, blk - SIDES * a.n_bc);
     }
 }
 
@@ -495,7 +618,7 @@ size_t dg_smem() { return (size_t)(8 * kQ + 2 * kQ + 4 * kQ) * sizeof(float) + (
 template <typename T, int P, int N>
 size_t off_smem(bool side_c) { return (size_t)(8 * kQ + 2 * kQ) * sizeof(float) + ((size_t)(kQ + N) * lds_ld<T>(P) + ((side_c && off_c_in_lds<T, P, N>()) ? (size_t)kQ * lds_ld<T>(N) : 0)) * sizeof(T); }
 template <typename T, int N>
-size_t bcf_smem() { return (size_t)(kQ + N) * lds_ld<T>(kQ) * sizeof(T); }
+size_t bcf_smem() { return sizeof(T) == 2 ? (size_t)2 * kQ * kQ * sizeof(T) : (size_t)(kQ + N) * lds_ld<T>(kQ) * sizeof(T); }
 
 template <typename T, int P, int N>
 int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
@@ -649,7 +772,10 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
             else if (n_ss > 0) slice_sum_kernel<<<(unsigned)n_ss, 256, 0, st>>>(sa);
         }
         if ((rc = check_launch("ssd tail1_kernel"))) return rc;
-        auto k = tail2_kernel<T, N>;
+        // 16-bit operands: one workgroup per (batch, chunk, group) once those alone fill the chip, one per side below that
+        const bool both = sizeof(T) == 2 && ngrp >= kTail2BothFrom;
+        auto k = tail2_kernel<T, N, false>;
+        if constexpr (sizeof(T) == 2) { if (both) k = tail2_kernel<T, N, true>; }
         const size_t sm = bcf_smem<T, N>();
         if ((rc = allow_smem(k, sm))) return rc;
         Tail2Args ta;
@@ -659,7 +785,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
         ta.dAp = w.dAp; ta.dDp = w.dDp; ta.dbp = w.dbp; ta.dA = p->dA; ta.dD = p->D ? p->dD : nullptr;
         ta.dbias = p->dt_bias ? p->d_dt_bias : nullptr;
         ta.seqlen = p->seqlen; ta.ngroups = p->ngroups; ta.nchunks = nc; ta.batch = p->batch; ta.nheads = p->nheads; ta.n_bc = ngrp;
-        k<<<(unsigned)(2 * ngrp + p->nheads), 512, sm, st>>>(ta);
+        k<<<(unsigned)((both ? 1 : 2) * ngrp + p->nheads), 512, sm, st>>>(ta);
         if ((rc = check_launch("ssd tail2_kernel"))) return rc;
     }
     return M2_OK;

@@ -31,6 +31,7 @@ CASES = [
     (1, 640, 2, 128, 128, 2),    # p = 128 over an odd number of chunks (the state pass peels one off)
     (1, 512, 4, 128, 64, 1),     # p = 128, n = 64 over an even number
     (2, 896, 4, 64, 64, 2),      # n = 64: two-wave state pass, seven chunks
+    (2, 2000, 8, 64, 64, 8),     # 256 (batch, chunk, group) triples: the group finish takes both sides per workgroup; ragged
 ]
 
 
