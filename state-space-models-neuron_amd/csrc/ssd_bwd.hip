@@ -35,7 +35,7 @@
 //                             per (b, chunk, group, head slice)  dx, per-token decay-gradient terms, e^{Lam} <dS, S_prev>,
 //                                                                dD partials, partial state parts of dB / dC
 //   tail1_kernel              da_body: ddt, dA partials per (b, head, chunk);  slice_sum_body: partials over the head slices
-//   tail2_kernel              bc_final_body per (b, chunk, group): dC = dG B + dCoff, dB = dG^T C + dBoff;
+//   tail2_kernel              bc_final16_body [bc_final_body] per (b, chunk, group): dC = dG B + dCoff, dB = dG^T C + dBoff;
 //                             ad_reduce_body per head: dA, dD (fixed order, no atomics)
 #include "ssd_host.hpp"
 
@@ -341,24 +341,8 @@ tail1_kernel(const DaArgs d, const int64_t n_da, const SliceSumArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------
-// acc[0][j] += A[rows 0..31, k0:k1] * M[column blocks nb0 + j, k0:k1]^T with A in LDS (row-major) and M a transposed
-// B / C tile in MFMA operand order (mt_offset), copied to LDS as it lies: a wave's B-operand fragment is one
-// contiguous KiB.
-template <int NB, typename T>
-__device__ __forceinline__ void wave_mma_mt(floatx16 (&acc)[1][NB], const T* __restrict__ A, int lda, const T* __restrict__ Mt,
-                                            int nb0, int k0, int k1) {
-    const int lane = threadIdx.x & 63;
-    const int r = lane & 31, kh = (lane >> 5) * 8;
-    for (int k = k0; k < k1; k += 16) {
-        const Frag<T> af = load_frag(A + r * lda + k + kh);
-#pragma unroll
-        for (int j = 0; j < NB; ++j) mma_frag(acc[0][j], af, load_frag(Mt + (((nb0 + j) * (kQ / 16) + (k >> 4)) * 64 + lane) * 8));
-    }
-}
-
-// Group-level finish, one side per workgroup of 512 threads:  dC = dG B + sum dCoff  or  dB = dG^T C + sum dBoff  (dG and
-// the off parts already summed over the head slices).  The head-summed dG is rounded to the operand type only here; for
-// bf16 it is split into hi + lo (two MFMA passes) so the contractions see it at ~2^-17 relative.
+// Group-level finish for fp32 operands, one side per workgroup of 512 threads:  dC = dG B + sum dCoff  or
+// dB = dG^T C + sum dBoff  (dG and the off parts already summed over the head slices).
 template <typename T, int N>
 __device__ __forceinline__ void
 bc_final_body(const float* __restrict__ dGp, const float* __restrict__ dCp, const float* __restrict__ dBp,
@@ -366,6 +350,7 @@ bc_final_body(const float* __restrict__ dGp, const float* __restrict__ dCp, cons
               int64_t seqlen, int64_t ngroups, int64_t nchunks,
               int64_t dBsb, int64_t dBsl, int64_t dBsg, int64_t dCsb, int64_t dCsl, int64_t dCsg, int64_t c, int64_t g, int64_t b,
               const bool side_b) {
+    static_assert(sizeof(T) == 4, "16-bit operands take bc_final16_body");
     constexpr int LDQ = lds_ld<T>(kQ);
     constexpr int NB = N / 64;
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -394,32 +379,20 @@ bc_final_body(const float* __restrict__ dGp, const float* __restrict__ dCp, cons
             for (int jn = 0; jn < NB; ++jn) acc[0][jn][v] = op[row * N + (nb0 + jn) * 32 + r];
         }
     }
-    constexpr int NPASS = sizeof(T) == 2 ? 2 : 1;
     //   dC[i][n] += sum_{j<=i} dG[i][j] B[j][n]      (A = dG,   k = j in [0, 32 (rb + 1)) )
     //   dB[j][n] += sum_{i>=j} dG[i][j] C[i][n]      (A = dG^T, k = i in [32 rb, kQ) )
     const T* tile = (side_b ? Ct : Bt) + grp * (int64_t)(N * kQ);
-    if constexpr (sizeof(T) == 2) {
-        for (int e = tid; e < N * kQ / 8; e += 512) *reinterpret_cast<uint4*>(sT2 + e * 8) = *reinterpret_cast<const uint4*>(tile + e * 8);
-    } else {
-        stage_rows<T, N, kQ, 512, false>(sT2, LDQ, tile, kQ, N, nullptr, tid);
-    }
+    stage_rows<T, N, kQ, 512, false>(sT2, LDQ, tile, kQ, N, nullptr, tid);
     const int k0 = side_b ? rb * 32 : 0, k1 = side_b ? kQ : (rb + 1) * 32;
 #pragma unroll
-    for (int pass = 0; pass < NPASS; ++pass) {
+    for (int jb = 0; jb < 2; ++jb)
 #pragma unroll
-        for (int jb = 0; jb < 2; ++jb)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int i = rb * 32 + acc_row(lane, v), j = (cb0 + jb) * 32 + r;
-                const float full = dG[0][jb][v];
-                const T hi = from_f32<T>(full);
-                sA2[side_b ? j * LDQ + i : i * LDQ + j] = pass == 0 ? hi : from_f32<T>(full - to_f32(hi));
-            }
-        __syncthreads();
-        if constexpr (sizeof(T) == 2) wave_mma_mt<NB>(acc, sA2 + rb * 32 * LDQ, LDQ, sT2, nb0, k0, k1);
-        else wave_mma<1, NB>(acc, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, k0, k1);
-        __syncthreads();
-    }
+        for (int v = 0; v < 16; ++v) {
+            const int i = rb * 32 + acc_row(lane, v), j = (cb0 + jb) * 32 + r;
+            sA2[side_b ? j * LDQ + i : i * LDQ + j] = dG[0][jb][v];
+        }
+    __syncthreads();
+    wave_mma<1, NB>(acc, sA2 + rb * 32 * LDQ, LDQ, sT2 + nb0 * 32 * LDQ, LDQ, k0, k1);
     T* out = side_b ? dB + b * dBsb + t0 * dBsl + g * dBsg : dC + b * dCsb + t0 * dCsl + g * dCsg;
     const int64_t osl = side_b ? dBsl : dCsl;
 #pragma unroll
@@ -591,14 +564,15 @@ tail2_kernel(const Tail2Args a) {
     if (blk < SIDES * a.n_bc) {
         const int64_t q = blk / SIDES;
         const int64_t c = q % a.nchunks, g = (q / a.nchunks) % a.ngroups, b = q / (a.nchunks * a.ngroups);
-        if constexpr (sizeof(T) == 2)
+        if constexpr (sizeof(T) == 2) {
             bc_final16_body<T, N, BOTH>(a.dGp, a.dCp, a.dBp, static_cast<const T*>(a.Bt), static_cast<const T*>(a.Ct), static_cast<T*>(a.dB),
                                         static_cast<T*>(a.dC), a.seqlen, a.ngroups, a.nchunks, a.dBsb, a.dBsl, a.dBsg, a.dCsb, a.dCsl, a.dCsg, c, g,
                                         b, (blk & 1) != 0);
-        else
+        } else {
             bc_final_body<T, N>(a.dGp, a.dCp, a.dBp, static_cast<const T*>(a.Bt), static_cast<const T*>(a.Ct), static_cast<T*>(a.dB),
                                 static_cast<T*>(a.dC), a.seqlen, a.ngroups, a.nchunks, a.dBsb, a.dBsl, a.dBsg, a.dCsb, a.dCsl, a.dCsg, c, g, b,
                                 (blk & 1) != 0);
+        }
     } else {
         ad_reduce_body(a.dAp, a.dDp, a.dbp, a.dA, a.dD, a.dbias, a.batch, a.nheads, a.nchunks, blk - SIDES * a.n_bc);
     }
