@@ -101,6 +101,11 @@ template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float 
 // half of the wave (v_permlane32_swap).  With the transposed 32x32 accumulator layout (a lane and its partner hold the two
 // halves of each 8-element group of one row) this leaves every lane with whole groups of 8 consecutive elements.
 // (The scalars are passed by value on purpose: a bit cast applied directly to a vector element reads element 0.)
+__device__ __forceinline__ void pair_swap(uint32_t a, uint32_t b, uint32_t& lo, uint32_t& hi) {
+    const auto sw = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+    lo = sw[0];
+    hi = sw[1];
+}
 __device__ __forceinline__ void pair_swap(float a, float b, float& lo, float& hi) {
     const uint32_t ua = __builtin_bit_cast(uint32_t, a), ub = __builtin_bit_cast(uint32_t, b);
     const auto sw = __builtin_amdgcn_permlane32_swap(ua, ub, false, false);

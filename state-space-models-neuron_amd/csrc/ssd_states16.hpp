@@ -186,9 +186,15 @@ state_pass16_kernel(const StatePassArgs a) {
 #pragma unroll
             for (int j = 0; j < NBW; ++j)
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const uint2 w = {pack2<T>(acc[i][j][4 * q], acc[i][j][4 * q + 1]), pack2<T>(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3])};
-                    *reinterpret_cast<uint2*>(cO + (i * 32 + r) * LDO + n0 + j * 32 + 8 * q + 4 * half) = w;
+                for (int qp = 0; qp < 2; ++qp) {
+                    // a lane and its partner (lane ^ 32) hold the two halves of every 8-column group: one exchange of the packed
+                    // words leaves each with a whole group, written as 16 bytes (8-byte writes of 32 rows at this pitch would
+                    // meet pairwise in the same banks)
+                    const int q0 = 2 * qp, q1 = q0 + 1;
+                    uint32_t o0, o1, o2, o3;
+                    pair_swap(pack2<T>(acc[i][j][4 * q0], acc[i][j][4 * q0 + 1]), pack2<T>(acc[i][j][4 * q1], acc[i][j][4 * q1 + 1]), o0, o2);
+                    pair_swap(pack2<T>(acc[i][j][4 * q0 + 2], acc[i][j][4 * q0 + 3]), pack2<T>(acc[i][j][4 * q1 + 2], acc[i][j][4 * q1 + 3]), o1, o3);
+                    *reinterpret_cast<u32x4*>(cO + (i * 32 + r) * LDO + n0 + j * 32 + 8 * (q0 + half)) = u32x4{o0, o1, o2, o3};
                 }
         __syncthreads();          // both tiles are complete; every wave is done with the other buffers
         // the rows two chunks on (past the end: the last chunk once more, rather than branching around the loads)
