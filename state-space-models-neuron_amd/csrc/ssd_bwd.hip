@@ -316,8 +316,9 @@ off_kernel(const T* __restrict__ Arow, int64_t Asb, int64_t Asl, int64_t Ash,   
 // `tile` floats per (group, slice) tile; segment k covers threads [first_k, first_{k+1}).
 struct SliceSumSeg { const float* part; float* out; int64_t nslices, tile, first; };
 struct SliceSumArgs { SliceSumSeg seg[3]; int nseg; int64_t total; };
+template <int THREADS>
 __device__ __forceinline__ void slice_sum_body(const SliceSumArgs& a, int64_t blk) {
-    const int64_t idx = blk * 256 + threadIdx.x;
+    const int64_t idx = blk * THREADS + threadIdx.x;
     if (idx >= a.total) return;
     int k = 0;
     if (a.nseg > 1 && idx >= a.seg[1].first) k = 1;
@@ -330,14 +331,14 @@ __device__ __forceinline__ void slice_sum_body(const SliceSumArgs& a, int64_t bl
     *reinterpret_cast<floatx4*>(sg.out + grp * sg.tile + e) = s;
 }
 __global__ void __launch_bounds__(256)
-slice_sum_kernel(const SliceSumArgs a) { slice_sum_body(a, blockIdx.x); }
+slice_sum_kernel(const SliceSumArgs a) { slice_sum_body<256>(a, blockIdx.x); }
 // The slice sums and the per-chunk decay-gradient scan (da_body) in one launch: they are independent, and both are short.
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kDaHeads * 64)
 tail1_kernel(const DaArgs d, const int64_t n_da, const SliceSumArgs a) {
     const int64_t blk = blockIdx.x;
     if (blk < n_da) da_body<T>(d, blk);
-    else slice_sum_body(a, blk - n_da);
+    else slice_sum_body<kDaHeads * 64>(a, blk - n_da);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -716,7 +717,7 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
             da.dirp = w.dirp; da.rbp = w.rbp; da.dDp8 = w.dDp8;
             da.ddt = p->ddt; da.dt_f32 = dt_f32; da.ddt_sb = p->ddt_stride_b; da.ddt_sl = p->ddt_stride_l; da.dAp = w.dAp; da.dDp = w.dDp;
             da.dbp = p->dt_bias ? w.dbp : nullptr;
-            da.seqlen = p->seqlen; da.nheads = p->nheads; da.nchunks = nc; da.total = p->batch * p->nheads * nc;
+            da.seqlen = p->seqlen; da.nheads = p->nheads; da.nchunks = nc; da.batch = p->batch;
         } else {
             auto k = diag_off_kernel<T, P, N, true>;
             const size_t sm = diag_smem<T, P, N, true>();
@@ -741,9 +742,12 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
             add(w.dCp, w.dCs, w.ns_c, (int64_t)kQ * N, &cs);
             add(w.dBp, w.dBs, w.ns_b, (int64_t)kQ * N, &bs);
             sa.total = first;
-            const int64_t n_ss = ceil_div(first, (int64_t)256), n_da = have_da ? ceil_div(da.total, (int64_t)4) : 0;
-            if (have_da) tail1_kernel<T><<<(unsigned)(n_da + n_ss), 256, 0, st>>>(da, n_da, sa);
-            else if (n_ss > 0) slice_sum_kernel<<<(unsigned)n_ss, 256, 0, st>>>(sa);
+            if (have_da) {
+                const int64_t n_da = da_blocks(da), n_ss = ceil_div(first, (int64_t)(kDaHeads * 64));
+                tail1_kernel<T><<<(unsigned)(n_da + n_ss), kDaHeads * 64, 0, st>>>(da, n_da, sa);
+            } else if (first > 0) {
+                slice_sum_kernel<<<(unsigned)ceil_div(first, (int64_t)256), 256, 0, st>>>(sa);
+            }
         }
         if ((rc = check_launch("ssd tail1_kernel"))) return rc;
         // 16-bit operands: one workgroup per (batch, chunk, group) once those alone fill the chip, one per side below that

@@ -429,76 +429,110 @@ ssd_bwd16_kernel(const Bwd16Args a) {
 }
 
 // Per (batch, head, chunk): da_t = sum_{i>=t} (dl_diag_i + dl_c_i) + sum_{j<t} rb_j + dlam,  ddt_t = A da_t + dir_t,
-// dA partial = sum_t da_t dt_t, dD partial = sum of the per-wave partials.  One wave per (b, h, c), four per
-// workgroup (the first four waves of workgroup `blk` of tail1_kernel); lanes hold the tokens in reverse order (127 - lane, 63 - lane), so the suffix over tokens is an inclusive
-// prefix over lanes and the exclusive prefix over tokens an exclusive suffix over lanes.
+// dA partial = sum_t da_t dt_t, dD partial = sum of the per-wave partials.  One wave per (b, h, c); lanes hold the tokens in
+// reverse order (127 - lane, 63 - lane), so the suffix over tokens is an inclusive prefix over lanes and the exclusive prefix
+// over tokens an exclusive suffix over lanes.  The kDaHeads waves of a workgroup (workgroup `blk` of tail1_kernel) take
+// consecutive heads of one (batch, chunk): ddt is [b][l][h], so their results for a token are neighbours in memory and
+// leave through LDS as one 16-byte (operand type) or two 16-byte (fp32) stores per token instead of one 2- or 4-byte
+// store per token and head.
+constexpr int kDaHeads = 8;
 struct DaArgs {
     const float* ldtab; const float* A; const float* dl_diag; const float* dl_c; const float* dlam;
     const float* dirp; const float* rbp; const float* dDp8;
     void* ddt; int dt_f32; int64_t ddt_sb, ddt_sl; float* dAp; float* dDp;
     float* dbp;            // with softplus folded into the scan: [b][h][c] partials of d_dt_bias, and ddt is w.r.t. the raw dt; else null
-    int64_t seqlen, nheads, nchunks, total;
+    int64_t seqlen, nheads, nchunks, batch;
 };
+inline int64_t da_blocks(const DaArgs& q) { return q.batch * q.nchunks * ((q.nheads + kDaHeads - 1) / kDaHeads); }
 template <typename T>
 __device__ __forceinline__ void da_body(const DaArgs& q, int64_t blk) {
     const float* __restrict__ ldtab = q.ldtab; const float* __restrict__ A = q.A;
     const float* __restrict__ dl_diag = q.dl_diag; const float* __restrict__ dl_c = q.dl_c; const float* __restrict__ dlam = q.dlam;
     const float* __restrict__ dirp = q.dirp; const float* __restrict__ rbp = q.rbp; const float* __restrict__ dDp8 = q.dDp8;
-    void* __restrict__ ddt = q.ddt; const int dt_f32 = q.dt_f32; const int64_t ddt_sb = q.ddt_sb, ddt_sl = q.ddt_sl;
+    const int dt_f32 = q.dt_f32; const int64_t ddt_sb = q.ddt_sb, ddt_sl = q.ddt_sl;
     float* __restrict__ dAp = q.dAp; float* __restrict__ dDp = q.dDp; float* __restrict__ dbp = q.dbp;
-    const int64_t seqlen = q.seqlen, nheads = q.nheads, nchunks = q.nchunks, total = q.total;
-    const int lane = threadIdx.x & 63;
-    const int64_t bhc = blk * 4 + (threadIdx.x >> 6);
-    if (bhc >= total) return;
-    const int64_t c = bhc % nchunks, h = (bhc / nchunks) % nheads, b = bhc / (nchunks * nheads);
+    const int64_t seqlen = q.seqlen, nheads = q.nheads, nchunks = q.nchunks;
+    __shared__ float sv[kDaHeads][kQ];      // ddt of the workgroup's heads, [head][token]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t hgroups = (nheads + kDaHeads - 1) / kDaHeads;
+    const int64_t hg = blk % hgroups, c = (blk / hgroups) % nchunks, b = blk / (hgroups * nchunks);
+    const int64_t h0 = hg * kDaHeads, h = h0 + wave;
     const int64_t t0 = c * kQ;
     const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
     const int ta = kQ - 1 - lane, tb = 63 - lane;
-    const float Ah = A[h];
-    float xa = dl_diag[bhc * kQ + ta] + dl_c[bhc * kQ + ta];
-    float xb = dl_diag[bhc * kQ + tb] + dl_c[bhc * kQ + tb];
-    const float ra = rbp[bhc * kQ + ta], rbv = rbp[bhc * kQ + tb];
-    const float dira = dirp[bhc * kQ + ta], dirb = dirp[bhc * kQ + tb];
-    const float dta = ldtab[bhc * 2 * kQ + kQ + ta], dtb = ldtab[bhc * 2 * kQ + kQ + tb];     // 0 past the end of the sequence
-    float dlm = 0.f;
+    if (h < nheads) {      // wave-uniform
+        const int64_t bhc = (b * nheads + h) * nchunks + c;
+        const float Ah = A[h];
+        float xa = dl_diag[bhc * kQ + ta] + dl_c[bhc * kQ + ta];
+        float xb = dl_diag[bhc * kQ + tb] + dl_c[bhc * kQ + tb];
+        const float ra = rbp[bhc * kQ + ta], rbv = rbp[bhc * kQ + tb];
+        const float dira = dirp[bhc * kQ + ta], dirb = dirp[bhc * kQ + tb];
+        const float dta = ldtab[bhc * 2 * kQ + kQ + ta], dtb = ldtab[bhc * 2 * kQ + kQ + tb];     // 0 past the end of the sequence
+        float dlm = 0.f;
 #pragma unroll
-    for (int sp = 0; sp < kDlamParts; ++sp) dlm += dlam[bhc * kDlamParts + sp];
-    float ya = ra, yb = rbv;
+        for (int sp = 0; sp < kDlamParts; ++sp) dlm += dlam[bhc * kDlamParts + sp];
+        float ya = ra, yb = rbv;
 #pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const float na = __shfl_up(xa, o, 64), nb = __shfl_up(xb, o, 64);
-        const float ma = __shfl_down(ya, o, 64), mb = __shfl_down(yb, o, 64);
-        if (lane >= o) { xa += na; xb += nb; }
-        if (lane + o < 64) { ya += ma; yb += mb; }
-    }
-    xb += __shfl(xa, 63, 64);
-    xa += (ya - ra) + __shfl(yb, 0, 64);
-    xb += yb - rbv;
-    const float da_a = xa + dlm, da_b = xb + dlm;
-    float dAl = 0.f, dbl = 0.f;
-    if (ta < valid) {
-        float val = Ah * da_a + dira;
-        if (dbp) { val *= softplus_grad_of_value(dta); dbl += val; }      // dta = softplus(raw dt + bias)
-        const int64_t oo = b * ddt_sb + (t0 + ta) * ddt_sl + h;
-        if (dt_f32) static_cast<float*>(ddt)[oo] = val; else static_cast<T*>(ddt)[oo] = from_f32<T>(val);
-        dAl += da_a * dta;
-    }
-    if (tb < valid) {
-        float val = Ah * da_b + dirb;
-        if (dbp) { val *= softplus_grad_of_value(dtb); dbl += val; }
-        const int64_t oo = b * ddt_sb + (t0 + tb) * ddt_sl + h;
-        if (dt_f32) static_cast<float*>(ddt)[oo] = val; else static_cast<T*>(ddt)[oo] = from_f32<T>(val);
-        dAl += da_b * dtb;
-    }
-    dAl = warp_sum(dAl);
-    if (dbp) dbl = warp_sum(dbl);
-    if (lane == 0) {
-        dAp[bhc] = dAl;
-        if (dbp) dbp[bhc] = dbl;
-        float s = 0.f;
+        for (int o = 1; o < 64; o <<= 1) {
+            const float na = __shfl_up(xa, o, 64), nb = __shfl_up(xb, o, 64);
+            const float ma = __shfl_down(ya, o, 64), mb = __shfl_down(yb, o, 64);
+            if (lane >= o) { xa += na; xb += nb; }
+            if (lane + o < 64) { ya += ma; yb += mb; }
+        }
+        xb += __shfl(xa, 63, 64);
+        xa += (ya - ra) + __shfl(yb, 0, 64);
+        xb += yb - rbv;
+        const float da_a = xa + dlm, da_b = xb + dlm;
+        float dAl = 0.f, dbl = 0.f;
+        float va = 0.f, vb = 0.f;
+        if (ta < valid) {
+            va = Ah * da_a + dira;
+            if (dbp) { va *= softplus_grad_of_value(dta); dbl += va; }      // dta = softplus(raw dt + bias)
+            dAl += da_a * dta;
+        }
+        if (tb < valid) {
+            vb = Ah * da_b + dirb;
+            if (dbp) { vb *= softplus_grad_of_value(dtb); dbl += vb; }
+            dAl += da_b * dtb;
+        }
+        sv[wave][ta] = va;
+        sv[wave][tb] = vb;
+        dAl = warp_sum(dAl);
+        if (dbp) dbl = warp_sum(dbl);
+        if (lane == 0) {
+            dAp[bhc] = dAl;
+            if (dbp) dbp[bhc] = dbl;
+            float s = 0.f;
 #pragma unroll
-        for (int w = 0; w < 8; ++w) s += dDp8[bhc * 8 + w];
-        dDp[bhc] = s;
+            for (int w = 0; w < 8; ++w) s += dDp8[bhc * 8 + w];
+            dDp[bhc] = s;
+        }
+    }
+    __syncthreads();
+    // one token per thread: its kDaHeads (fewer in the last head group) values are consecutive in ddt
+    const int t = threadIdx.x;
+    if (t < valid) {
+        const int hc = (int)(nheads - h0 < kDaHeads ? nheads - h0 : kDaHeads);
+        const int64_t oo = b * ddt_sb + (t0 + t) * ddt_sl + h0;
+        if (dt_f32) {
+            float* o = static_cast<float*>(q.ddt) + oo;
+            if (hc == kDaHeads && (reinterpret_cast<uintptr_t>(o) & 15) == 0) {
+                *reinterpret_cast<floatx4*>(o) = floatx4{sv[0][t], sv[1][t], sv[2][t], sv[3][t]};
+                *reinterpret_cast<floatx4*>(o + 4) = floatx4{sv[4][t], sv[5][t], sv[6][t], sv[7][t]};
+            } else {
+                for (int k = 0; k < hc; ++k) o[k] = sv[k][t];
+            }
+        } else {
+            T* o = static_cast<T*>(q.ddt) + oo;
+            if (hc == kDaHeads && (reinterpret_cast<uintptr_t>(o) & 15) == 0) {
+                T e[kDaHeads];
+#pragma unroll
+                for (int k = 0; k < kDaHeads; ++k) e[k] = from_f32<T>(sv[k][t]);
+                *reinterpret_cast<uint4*>(o) = *reinterpret_cast<const uint4*>(e);
+            } else {
+                for (int k = 0; k < hc; ++k) o[k] = from_f32<T>(sv[k][t]);
+            }
+        }
     }
 }
 
