@@ -187,9 +187,8 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
         pa.dt = p->dt; pa.dt_f32 = dt_f32; pa.dt_bias = p->dt_bias; pa.A = p->A; pa.ldtab = w.ldtab; pa.lam = w.lam;
         pa.dtsb = p->dt_stride_b; pa.dtsl = p->dt_stride_l;
         pa.seqlen = p->seqlen; pa.nheads = p->nheads; pa.ngroups = p->ngroups; pa.nchunks = nc;
-        pa.total_bhc = p->batch * p->nheads * nc;
         pa.n_cb = nc * p->ngroups * p->batch;
-        const int64_t blocks = kCbParts * pa.n_cb + ceil_div(pa.total_bhc, (int64_t)4);
+        const int64_t blocks = kCbParts * pa.n_cb + ld_table_blocks(p->batch, p->nheads, nc);
         M2_REQUIRE(blocks < ((int64_t)1 << 31), M2_ERR_SHAPE, "ssd: too many workgroups");
         k<<<(unsigned)blocks, 256, sm, st>>>(pa);
         if ((rc = check_launch("ssd prep_kernel"))) return rc;

@@ -116,22 +116,59 @@ cb_body(const T* __restrict__ Bm, const T* __restrict__ Cm, float* __restrict__ 
 }
 
 // ------------------------------------------------------------------------------------------
-// Cumulative log-decay table: one wave per (batch, head, chunk), four per workgroup; ldtab[bhc] = [ l[0..kQ) | dt[0..kQ) ] in fp32,
+// Cumulative log-decay table: one wave per (batch, head, chunk); ldtab[bhc] = [ l[0..kQ) | dt[0..kQ) ] in fp32,
 // l = inclusive cumsum of A_h dt within the chunk, lam[bhc] = l[kQ-1].  Every other kernel reads this table instead
-// of gathering dt (stride = nheads elements) and scanning it again per head.
+// of gathering dt (stride = nheads elements) and scanning it again per head.  The four waves of a workgroup take four
+// consecutive heads of one (batch, chunk): dt is [b][l][h], so a token's four values are 8 (fp32: 16) consecutive bytes
+// and are fetched by one thread per token and handed to the waves through LDS, instead of 128 two-byte gathers per wave.
+constexpr int kLdHeads = 4;
+inline int64_t ld_table_blocks(int64_t batch, int64_t nheads, int64_t nchunks) { return batch * nchunks * ((nheads + kLdHeads - 1) / kLdHeads); }
 template <typename T>
 __device__ __forceinline__ void
 ld_table_body(const void* __restrict__ dt, int dt_f32, const float* __restrict__ dt_bias, const float* __restrict__ A, float* __restrict__ ldtab,
-              float* __restrict__ lam, int64_t seqlen, int64_t nheads, int64_t nchunks, int64_t total,
+              float* __restrict__ lam, int64_t seqlen, int64_t nheads, int64_t nchunks,
               int64_t dtsb, int64_t dtsl, int64_t blk) {
-    const int lane = threadIdx.x & 63;
-    const int64_t bhc = blk * 4 + (threadIdx.x >> 6);
-    if (bhc >= total) return;
-    const int64_t c = bhc % nchunks, h = (bhc / nchunks) % nheads, b = bhc / (nchunks * nheads);
+    __shared__ float sdt[kLdHeads][kQ];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t hgroups = (nheads + kLdHeads - 1) / kLdHeads;
+    const int64_t hg = blk % hgroups, c = (blk / hgroups) % nchunks, b = blk / (hgroups * nchunks);
+    const int64_t h0 = hg * kLdHeads, h = h0 + wave;
     const int64_t t0 = c * kQ;
     const int valid = (int)((seqlen - t0) < kQ ? (seqlen - t0) : kQ);
-    float l0, l1, d0, d1;
-    wave_dt_load<T>(dt, dt_f32, b * dtsb + t0 * dtsl + h, dtsl, valid, d0, d1);
+    const int hc = (int)(nheads - h0 < kLdHeads ? nheads - h0 : kLdHeads);
+    if (threadIdx.x < kQ) {
+        const int t = threadIdx.x;
+        float v[kLdHeads] = {0.f, 0.f, 0.f, 0.f};      // tokens past the end of the sequence behave as dt = 0
+        if (t < valid) {
+            const int64_t off = b * dtsb + (t0 + t) * dtsl + h0;
+            if (dt_f32) {
+                const float* p = static_cast<const float*>(dt) + off;
+                if (hc == kLdHeads && (reinterpret_cast<uintptr_t>(p) & 15) == 0) {
+                    const floatx4 q = *reinterpret_cast<const floatx4*>(p);
+#pragma unroll
+                    for (int k = 0; k < kLdHeads; ++k) v[k] = q[k];
+                } else {
+                    for (int k = 0; k < hc; ++k) v[k] = p[k];
+                }
+            } else {
+                const T* p = static_cast<const T*>(dt) + off;
+                if (hc == kLdHeads && (reinterpret_cast<uintptr_t>(p) & (kLdHeads * sizeof(T) - 1)) == 0) {
+                    const RawVec<T, kLdHeads> q = *reinterpret_cast<const RawVec<T, kLdHeads>*>(p);
+                    const T* e = reinterpret_cast<const T*>(&q);
+#pragma unroll
+                    for (int k = 0; k < kLdHeads; ++k) v[k] = to_f32(e[k]);
+                } else {
+                    for (int k = 0; k < hc; ++k) v[k] = to_f32(p[k]);
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kLdHeads; ++k) sdt[k][t] = v[k];
+    }
+    __syncthreads();
+    if (h >= nheads) return;      // wave-uniform, behind the only barrier
+    const int64_t bhc = (b * nheads + h) * nchunks + c;
+    float l0, l1, d0 = sdt[wave][lane], d1 = sdt[wave][lane + 64];
     if (dt_bias) {
         // dt holds the raw projection: the step size is softplus(dt + dt_bias) (0 stays 0 past the end of the sequence)
         const float bh = dt_bias[h];
@@ -150,7 +187,7 @@ struct PrepArgs {
     const void* Bm; const void* Cm; float* Gf; void* Gm; void* Gmt; void* Bt; void* Ct;
     int64_t Bsb, Bsl, Bsg, Csb, Csl, Csg;
     const void* dt; int dt_f32; const float* dt_bias; const float* A; float* ldtab; float* lam; int64_t dtsb, dtsl;
-    int64_t seqlen, nheads, ngroups, nchunks, total_bhc, n_cb;
+    int64_t seqlen, nheads, ngroups, nchunks, n_cb;
 };
 template <typename T, int N>
 __global__ void __launch_bounds__(256)
@@ -163,7 +200,7 @@ prep_kernel(const PrepArgs a) {
                       static_cast<T*>(a.Bt), static_cast<T*>(a.Ct), a.seqlen, a.ngroups, a.nchunks,
                       a.Bsb, a.Bsl, a.Bsg, a.Csb, a.Csl, a.Csg, c, g, b, (int)(blk % kCbParts));
     } else {
-        ld_table_body<T>(a.dt, a.dt_f32, a.dt_bias, a.A, a.ldtab, a.lam, a.seqlen, a.nheads, a.nchunks, a.total_bhc, a.dtsb, a.dtsl, blk - kCbParts * a.n_cb);
+        ld_table_body<T>(a.dt, a.dt_f32, a.dt_bias, a.A, a.ldtab, a.lam, a.seqlen, a.nheads, a.nchunks, a.dtsb, a.dtsl, blk - kCbParts * a.n_cb);
     }
 }
 
