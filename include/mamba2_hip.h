@@ -93,6 +93,14 @@ int m2_conv1d_bwd(const m2_conv1d_params* p, void* stream);
  * dt (b,l,h), A (h) fp32, x (b,l,h,p), B,C (b,l,g,n), D (h) fp32 or NULL,
  * initial_state / final_state (b,h,p,n) fp32 contiguous or NULL, y (b,l,h,p).
  * Supported: p in {64,128}, n in {64,128}, h % g == 0, any l >= 0, any b >= 0.
+ * Alignment and strides (both dtypes; refused with M2_ERR_ALIGN / M2_ERR_SHAPE, never copied):
+ *   - x, B, C, y and, in the backward, dy, dx, dB, dC: base pointer 16-byte aligned and every
+ *     stride a multiple of 16 bytes (8 elements of bf16, 4 of fp32): rows are read and written as
+ *     16-byte vectors, the gradients too (so a slice of a packed gradient buffer must start at a
+ *     column that is a multiple of 8 / 4);
+ *   - token strides (x, B, C, dt, y, dy, dx, dB, dC, ddt) in [0, 2^21) elements: row offsets inside
+ *     a chunk are 32-bit sums of 24-bit products;
+ *   - workspace 256-byte aligned, chunk_states 16-byte aligned; batch, nheads <= 65535.
  * Backward takes the same inputs plus dy (y is unused) and writes
  * dx, ddt, dB, dC in the dtype of the matching input and dA (h), dD (h) in fp32,
  * already summed over the batch (the reference sums them in its wrapper,
@@ -173,7 +181,8 @@ int m2_decode_step(const m2_decode_params* p, void* stream);
  * (its decode kernel allocates fresh outputs per call, mamba2_kernel_inference.py:114-116).
  *   - limit: batch x conv channels <= 1 048 576 (batch 195 at the 2.7B width); beyond it M2_ERR_WORKSPACE.
  *   - allocates nothing; the array's device address is looked up on the first call per device (make that first call
- *     outside a graph capture).  Each GPU holds its own 4 MiB copy until the process ends.
+ *     outside a graph capture).  The CURRENT device (hipGetDevice) must be the one `stream` belongs to: the address is
+ *     kept per current-device index.  Each GPU holds its own 4 MiB copy until the process ends.
  *   - all calls on one GPU share that array: calls that overlap on one GPU (two streams, two threads) race; calls on
  *     one stream, or otherwise ordered, are safe.  Nothing in it has to start at zero (every call overwrites what it reads). */
 int m2_decode_step_static(const m2_decode_params* p, void* stream);

@@ -249,7 +249,14 @@ extern "C" int m2_decode_step(const m2_decode_params* p, void* stream) {
 extern "C" int m2_decode_step_static(const m2_decode_params* p, void* stream) {
     using namespace m2;
     M2_REQUIRE(p, M2_ERR_NULL, "decode_step_static: params is NULL");
-    const int64_t Cx = p->nheads * p->headdim + 2 * p->ngroups * p->dstate;
+    // each factor is bounded by the scratch size before the channel count is formed, so that the products cannot overflow;
+    // negative or zero dimensions fall through to the shared checks below
+    const int64_t lim = (int64_t)kStaticScratchFloats;
+    const bool sane = p->nheads >= 0 && p->headdim >= 0 && p->ngroups >= 0 && p->dstate >= 0 && p->batch >= 0;
+    M2_REQUIRE(!sane || (p->nheads <= lim && p->headdim <= lim && p->ngroups <= lim && p->dstate <= lim && p->batch <= lim),
+               M2_ERR_WORKSPACE, "decode_step_static: a dimension exceeds the built-in scratch of %zu floats; use m2_decode_step with a workspace",
+               kStaticScratchFloats);
+    const int64_t Cx = sane ? p->nheads * p->headdim + 2 * p->ngroups * p->dstate : 0;
     // sizes beyond the built-in scratch are refused here; every other check is the shared one below
     M2_REQUIRE(p->batch <= 0 || Cx <= 0 || (uint64_t)Cx <= kStaticScratchFloats / (uint64_t)p->batch, M2_ERR_WORKSPACE,
                "decode_step_static: batch %lld x %lld conv channels exceed the built-in scratch of %zu floats; use m2_decode_step with a workspace",
@@ -264,17 +271,17 @@ namespace m2 {
 namespace {
 
 int decode_step_impl(const m2_decode_params* p, float* act, size_t act_bytes, const char* who, void* stream) {
-    M2_REQUIRE(p->dtype == M2_F32 || p->dtype == M2_BF16, M2_ERR_DTYPE, "decode_step: bad dtype %d", p->dtype);
-    M2_REQUIRE(p->param_dtype == M2_F32 || p->param_dtype == M2_BF16, M2_ERR_DTYPE, "decode_step: bad param dtype %d", p->param_dtype);
-    M2_REQUIRE(p->batch >= 0 && p->nheads >= 0 && p->headdim >= 1 && p->dstate >= 1, M2_ERR_SHAPE, "decode_step: bad dimension");
+    M2_REQUIRE(p->dtype == M2_F32 || p->dtype == M2_BF16, M2_ERR_DTYPE, "%s: bad dtype %d", who, p->dtype);
+    M2_REQUIRE(p->param_dtype == M2_F32 || p->param_dtype == M2_BF16, M2_ERR_DTYPE, "%s: bad param dtype %d", who, p->param_dtype);
+    M2_REQUIRE(p->batch >= 0 && p->nheads >= 0 && p->headdim >= 1 && p->dstate >= 1, M2_ERR_SHAPE, "%s: bad dimension", who);
     M2_REQUIRE(p->ngroups >= 1 && p->nheads % p->ngroups == 0, M2_ERR_SHAPE, "decode_step: nheads %lld not divisible by ngroups %lld",
                (long long)p->nheads, (long long)p->ngroups);
-    M2_REQUIRE(p->k >= 1 && p->k <= 8, M2_ERR_SHAPE, "decode_step: conv kernel size %d not in [1,8]", p->k);
-    M2_REQUIRE(p->W >= p->k - 1 && p->W <= 8, M2_ERR_SHAPE, "decode_step: conv state width %d must be in [k-1, 8]", p->W);
-    M2_REQUIRE(p->batch <= 65535, M2_ERR_SHAPE, "decode_step: batch exceeds the grid limit 65535");
+    M2_REQUIRE(p->k >= 1 && p->k <= 8, M2_ERR_SHAPE, "%s: conv kernel size %d not in [1,8]", who, p->k);
+    M2_REQUIRE(p->W >= p->k - 1 && p->W <= 8, M2_ERR_SHAPE, "%s: conv state width %d must be in [k-1, 8]", who, p->W);
+    M2_REQUIRE(p->batch <= 65535, M2_ERR_SHAPE, "%s: batch exceeds the grid limit 65535", who);
     if (p->batch == 0 || p->nheads == 0) return M2_OK;
-    M2_REQUIRE(p->xBC && p->conv_w && p->S && p->dt && p->A && p->y, M2_ERR_NULL, "decode_step: xBC, conv_w, S, dt, A, y are required");
-    M2_REQUIRE(p->W == 0 || p->conv_state, M2_ERR_NULL, "decode_step: conv_state is required");
+    M2_REQUIRE(p->xBC && p->conv_w && p->S && p->dt && p->A && p->y, M2_ERR_NULL, "%s: xBC, conv_w, S, dt, A, y are required", who);
+    M2_REQUIRE(p->W == 0 || p->conv_state, M2_ERR_NULL, "%s: conv_state is required", who);
     const int64_t Cx = p->nheads * p->headdim + 2 * p->ngroups * p->dstate;
     const size_t need = (size_t)(p->batch * Cx) * sizeof(float);
     M2_REQUIRE(act && act_bytes >= need, M2_ERR_WORKSPACE, "%s: workspace %zu bytes < %zu needed", who, act_bytes, need);

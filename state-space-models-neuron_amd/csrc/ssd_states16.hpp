@@ -42,12 +42,15 @@ struct StatePassArgs {
 constexpr int kStatePassSplit = 2;
 // one wave per 32 state columns
 template <int N> constexpr int state_pass_threads() { return (N / 32) * 64; }
-template <int P, int N>
+template <int P, int N, bool HILO = false>
 constexpr size_t state_pass_smem() {
-    return (size_t)2 * kQ * (P / 2) * 2 + (size_t)2 * (P / 2) * (N + 8) * 2;
+    return (size_t)(HILO ? 2 : 1) * 2 * kQ * (P / 2) * 2 + (size_t)2 * (P / 2) * (N + 8) * 2;
 }
 
-template <typename T, int P, int N, bool REVERSE, bool DLAM = REVERSE>
+// HILO: the scaled rows are staged as TWO 16-bit tiles, the rounded value and the rounded remainder, and each k step takes
+// two products, so that the fp32 scale dt e^{Lam - l} reaches the accumulators with 16 significand bits instead of 8 (the
+// final state is an fp32 output; with one tile its error is that of the operand rounding, 2^-9 of every term).
+template <typename T, int P, int N, bool REVERSE, bool DLAM = REVERSE, bool HILO = false>
 __global__ void __launch_bounds__(state_pass_threads<N>(), (P == 64 ? (DLAM ? 2 : 3) : (DLAM ? 1 : 2)))
 state_pass16_kernel(const StatePassArgs a) {
     static_assert(sizeof(T) == 2, "16-bit operands only");
@@ -65,8 +68,9 @@ state_pass16_kernel(const StatePassArgs a) {
     constexpr int NSP = RW / RPP;                      // store passes
     static_assert(RW % RPP == 0, "whole store passes");
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    T* sX = reinterpret_cast<T*>(smem_raw);                                 // [2][kQ][P / 2], slots swizzled inside each row
-    T* sO = sX + 2 * kQ * PH;                                               // [2][P / 2][LDO]
+    constexpr int XT = HILO ? 2 : 1;                   // staged tiles per chunk
+    T* sX = reinterpret_cast<T*>(smem_raw);                                 // [2][XT][kQ][P / 2], slots swizzled inside each row
+    T* sO = sX + 2 * XT * kQ * PH;                                          // [2][P / 2][LDO]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 31, half = lane >> 5;
@@ -157,7 +161,7 @@ state_pass16_kernel(const StatePassArgs a) {
             case 2: __builtin_amdgcn_s_setprio(1); break;
             default: __builtin_amdgcn_s_setprio(0); break;
         }
-        T* cX = sX + buf * (kQ * PH);
+        T* cX = sX + buf * (XT * kQ * PH);
         __builtin_amdgcn_sched_barrier(0);      // keep this chunk's loads out of the previous chunk's MFMA phase (registers)
         load_same(c);
         // the values loaded one chunk ahead become visible to the optimiser here and no earlier: otherwise their
@@ -173,8 +177,19 @@ state_pass16_kernel(const StatePassArgs a) {
             const float sc = REVERSE ? s.d[it] * __expf(s.l[it]) : s.d[it] * __expf(s.lam - s.l[it]);
             // word-wise (two elements per 32-bit word), so that the loaded vectors stay four whole registers until here
             u32x4 o;
+            if constexpr (HILO) {
+                u32x4 o2;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) o[q] = pack2<T>(unpack_lo<T>(s.x[it][q]) * sc, unpack_hi<T>(s.x[it][q]) * sc);
+                for (int q = 0; q < 4; ++q) {
+                    const float v0 = unpack_lo<T>(s.x[it][q]) * sc, v1 = unpack_hi<T>(s.x[it][q]) * sc;
+                    o[q] = pack2<T>(v0, v1);
+                    o2[q] = pack2<T>(v0 - unpack_lo<T>(o[q]), v1 - unpack_hi<T>(o[q]));
+                }
+                *reinterpret_cast<u32x4*>(cX + kQ * PH + (row * SPR_X + (slot ^ tile_swz<SPR_X>(row))) * 8) = o2;
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) o[q] = pack2<T>(unpack_lo<T>(s.x[it][q]) * sc, unpack_hi<T>(s.x[it][q]) * sc);
+            }
             *reinterpret_cast<u32x4*>(cX + (row * SPR_X + (slot ^ tile_swz<SPR_X>(row))) * 8) = o;
         }
         const float dec = __expf(s.lam);
@@ -233,28 +248,33 @@ state_pass16_kernel(const StatePassArgs a) {
                 for (int v = 0; v < 16; ++v) acc[i][j][v] *= dec;
         // all A-operand fragments of the chunk are read from LDS first: the eight products form one dependent chain, and a
         // read issued next to its product would put an LDS round trip between any two of them
-        Frag<T> af[PBW][8];
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-            const int ta = ks * 16 + tr_tok, tb = ta + 4;
+        for (int xt = 0; xt < XT; ++xt) {
+            const T* tX = cX + xt * (kQ * PH);
+            Frag<T> af[PBW][8];
 #pragma unroll
-            for (int i = 0; i < PBW; ++i) {
-                const int col = i * 32 + tr_col;
-                const tvec4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-                    (M2_LDS tvec4*)(cX + (ta * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(ta))) * 8 + (col & 7)));
-                const tvec4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-                    (M2_LDS tvec4*)(cX + (tb * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(tb))) * 8 + (col & 7)));
+            for (int ks = 0; ks < 8; ++ks) {
+                const int ta = ks * 16 + tr_tok, tb = ta + 4;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { af[i][ks].v[e] = lo[e]; af[i][ks].v[4 + e] = hi[e]; }
+                for (int i = 0; i < PBW; ++i) {
+                    const int col = i * 32 + tr_col;
+                    const tvec4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                        (M2_LDS tvec4*)(tX + (ta * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(ta))) * 8 + (col & 7)));
+                    const tvec4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                        (M2_LDS tvec4*)(tX + (tb * SPR_X + ((col >> 3) ^ tile_swz<SPR_X>(tb))) * 8 + (col & 7)));
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) { af[i][ks].v[e] = lo[e]; af[i][ks].v[4 + e] = hi[e]; }
+                }
             }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+                for (int i = 0; i < PBW; ++i)
+#pragma unroll
+                    for (int j = 0; j < NBW; ++j) mma_frag(acc[i][j], bf[j][ks], af[i][ks]);
+            if (XT > 1) __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks)
-#pragma unroll
-            for (int i = 0; i < PBW; ++i)
-#pragma unroll
-                for (int j = 0; j < NBW; ++j) mma_frag(acc[i][j], bf[j][ks], af[i][ks]);
     };
 
     // Chunks are taken two per loop iteration (one per register set); an odd first chunk is peeled off in front so that

@@ -123,6 +123,11 @@ ssd_y16_kernel(const DiagArgs a) {
     constexpr int SPR_S = N / 8, SPR_X = P / 8;            // 16-byte slots per row
     constexpr int NS = P * SPR_S / 256, NX = kQ * SPR_X / 256;   // direct-to-LDS loads per lane per tile
     constexpr int TAB = kQ + 32;
+    // y stores a wave issues per head in a full chunk: a lane stores its half of the 8-channel groups of its token, 16 bytes each.  The
+    // epilogue's loops run over exactly these bounds and the tile wait below leaves exactly this many operations in
+    // flight, so the two cannot drift apart.
+    constexpr int QPAIRS = 2, kStoresPerHead = BN * QPAIRS;
+    static_assert(kStoresPerHead * 16 == P, "a token row is stored by a lane pair, 8 channels per store");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* sS = reinterpret_cast<T*>(smem_raw);                       // [2][P][N]     swizzled slots
     T* sX = sS + 2 * P * N;                                       // [2][kQ][P]    swizzled slots
@@ -196,8 +201,8 @@ ssd_y16_kernel(const DiagArgs a) {
 
         // this wave's share of the tiles of head hh, and the whole [ l | dt ] table, have landed.  The y stores of the head
         // before were issued behind these copies and vector-memory operations retire in issue order, so in a full chunk
-        // (every lane stores, 2 BN instructions per head) they may stay in flight across the wait
-        if (hh > 0 && valid == kQ) wait_vmem_keep<2 * BN>(1); else wait_vmem_all();
+        // (every lane stores, kStoresPerHead instructions per head) they may stay in flight across the wait
+        if (hh > 0 && valid == kQ) wait_vmem_keep<kStoresPerHead>(1); else wait_vmem_all();
         // ---- wave-private decay tables from the shared [ l | dt ] table
         const float* sl = sLD + buf * 2 * kQ;
         const float* sd = sl + kQ;
@@ -285,7 +290,7 @@ ssd_y16_kernel(const DiagArgs a) {
 #pragma unroll
         for (int j = 0; j < BN; ++j) {
 #pragma unroll
-            for (int qp = 0; qp < 2; ++qp) {
+            for (int qp = 0; qp < QPAIRS; ++qp) {
                 float g8[8];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {

@@ -10,8 +10,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# M2_LIB overrides the library path (used to compare builds of the same ABI)
-LIB_PATH = os.environ.get("M2_LIB") or os.path.join(_HERE, "libmamba2_hip.so")
+LIB_PATH = os.path.join(_HERE, "libmamba2_hip.so")
 
 M2_F32, M2_BF16 = 0, 1
 ACT = {None: 0, "identity": 0, "silu": 1, "swish": 1, "relu": 2}
@@ -100,16 +99,20 @@ SYMBOLS = {
 _lib = None
 
 
-def load():
-    """Load the library once.  Raises RuntimeError when it has not been built."""
+def load(path=None):
+    """Load the library once.  Raises RuntimeError when it has not been built.  ``path`` names another build of the same
+    ABI (it must be given on the first call of the process: the library that is loaded first stays)."""
     global _lib
     if _lib is not None:
+        if path is not None and os.path.abspath(path) != _lib._name:
+            raise RuntimeError(f"{_lib._name} is already loaded; cannot switch to {path}")
         return _lib
-    if not os.path.exists(LIB_PATH):
+    path = os.path.abspath(path) if path is not None else LIB_PATH
+    if not os.path.exists(path):
         raise RuntimeError(
-            f"{LIB_PATH} is missing: build it with `python state-space-models-neuron_amd/build.py` "
+            f"{path} is missing: build it with `python state-space-models-neuron_amd/build.py` "
             "(there is no fallback path; the HIP extension is required)")
-    lib = C.CDLL(LIB_PATH)
+    lib = C.CDLL(path)
     for name, (res, args) in SYMBOLS.items():
         fn = getattr(lib, name)
         fn.restype = res

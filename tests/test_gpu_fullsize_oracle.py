@@ -7,8 +7,8 @@
       step, every layer with its own states, each checked against the oracle.
 
 The bar is the stated one: fp32 results max|err| / max|ref| <= 1e-4; bf16 computations max|err| <= 2e-2 x RMS(ref) on the
-RAW error, plus, for a tensor stored in bf16, what storing the exact value costs (conftest.rel_rms_err; every raw figure
-is logged).  Inputs follow the reference's parity script (mamba2_kernel.py:555-564) as the configurations state them.
+RAW error; a tensor stored in bf16 whose raw figure is over the bar is allowed what storing the exact value in bf16
+costs, given a relative L2 error under 1e-2 (conftest.rel_rms_err; every raw figure is logged).  Inputs follow the reference's parity script (mamba2_kernel.py:555-564) as the configurations state them.
 """
 import math
 
@@ -38,9 +38,9 @@ def test_ssd_fwd_bwd_against_oracle_full_size(b, l, h, p, n, g):
            "dB": lv["B"].grad, "dC": lv["C"].grad, "dD": lv["D"].grad}
     bad = {}
     for k, v in got.items():
-        # y, dx, ddt, dB, dC leave in bf16; the final state and dA are fp32 sums of MFMA products whose operands (the
-        # decay-weighted dt x rows) were rounded to bf16: the error of an element is proportional to its own magnitude
-        e = rel_rms_err(v.cpu(), ref[k], name=k, bf16_operands=True)
+        # y, dx, ddt, dB, dC leave in bf16 (storage floor once the raw figure is over the bar); the final state, dA and dD are
+        # fp32 results and are held to the raw bar
+        e = rel_rms_err(v.cpu(), ref[k], name=k)
         l2 = ((v.double().cpu() - ref[k]).norm() / ref[k].norm()).item()
         if not (e < 2e-2 and l2 < 1e-2):
             bad[k] = (e, l2)
@@ -103,3 +103,67 @@ def test_decode_step_against_oracle_c4(layers):
         assert rel_err(state[i][2].cpu(), S_ref) < 1e-4, i
         # y leaves in bf16
         assert rel_rms_err(y.cpu(), y_ref, name=f"y[layer {i}]" if i < 2 else None) < 2e-2, i
+
+
+def test_fused_core_against_oracle_c3():
+    """The fused mixer core zxBCdt -> norm_out of the 7B layer (BASELINE configuration 3: b2 l4096, d_inner 8192, 128 heads,
+    8 groups, state 128), forward and backward, against oracle.mixer.fused_core_ref in fp64.  The chain hands bf16 tensors
+    from stage to stage; the floor of those hand-overs is measured with the same oracle and a bf16 round at each
+    (as tests/test_gpu_mixer.py does at small widths), and the relative L2 error is held to 1e-2."""
+    from conftest import raw_rms_err
+    from mamba2.fused_kernel import mamba2_fused_kernel
+    from oracle.mixer import fused_core_ref
+    b, l, h, p, n, g = 2, 4096, 128, 64, 128, 8
+    d_inner = h * p
+    width = 2 * d_inner + 2 * g * n + h
+    gen = torch.Generator().manual_seed(5)
+    zx = torch.randn(b, l, width, generator=gen)
+    zx[..., 2 * d_inner:2 * d_inner + 2 * g * n] /= n ** 0.5
+    t = {"zxBCdt": zx.to(torch.bfloat16), "A": -torch.exp(torch.empty(h).uniform_(0.0, 2.77, generator=gen)),
+         "D": torch.ones(h) + 0.1 * torch.randn(h, generator=gen),
+         "conv_w": (torch.rand(d_inner + 2 * g * n, 1, 4, generator=gen) - 0.5).to(torch.bfloat16),
+         "conv_b": (torch.rand(d_inner + 2 * g * n, generator=gen) - 0.5).to(torch.bfloat16),
+         "dt_bias": torch.empty(h).uniform_(-5.0, -2.0, generator=gen), "norm_w": 1.0 + 0.1 * torch.randn(d_inner, generator=gen)}
+    dout = torch.randn(b, l, d_inner, generator=gen).to(torch.bfloat16)
+    names = ("zxBCdt", "A", "D", "conv_w", "conv_b", "dt_bias", "norm_w")
+    torch.set_num_threads(min(16, torch.get_num_threads()))
+
+    class RoundBF16(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x):
+            return x.bfloat16().to(x.dtype)
+
+        @staticmethod
+        def backward(ctx, gr):
+            return gr.bfloat16().to(gr.dtype)
+
+    def oracle(handover):
+        lv = {k: t[k].double().clone().requires_grad_(True) for k in names}
+        zin = lv["zxBCdt"] if handover is None else handover(lv["zxBCdt"])
+        out = fused_core_ref(zin, lv["A"], lv["D"], lv["conv_w"], lv["conv_b"], lv["dt_bias"], lv["norm_w"], g, n, d_inner, p, handover=handover)
+        out.backward(dout.double())
+        return {"norm_out": out.detach(), **{"d" + k: lv[k].grad for k in names}}
+
+    ref = oracle(None)
+    floor = oracle(RoundBF16.apply)
+    lv = {k: t[k].to(DEV).clone().requires_grad_(True) for k in names}
+    out = mamba2_fused_kernel(*(lv[k] for k in names), g, n, d_inner, p)
+    out.backward(dout.to(DEV))
+    got = {"norm_out": out.detach(), **{"d" + k: lv[k].grad for k in names}}
+    parts = [d_inner, d_inner, g * n, g * n, h]          # the packed gradient holds quantities of different scale
+    bad = {}
+
+    def check(k, a, r, f):
+        e_floor = raw_rms_err(f, r)
+        e = rel_rms_err(a.cpu(), r, name=k, extra_floor=e_floor)
+        l2 = ((a.double().cpu() - r).norm() / r.norm()).item()
+        if not (e < 2e-2 and l2 < 1e-2):
+            bad[k] = (e, e_floor, l2)
+
+    for k in got:
+        if k == "dzxBCdt":
+            for nm, a, r, f in zip(("dz", "dx", "dB", "dC", "ddt"), *(torch.split(q[k], parts, dim=-1) for q in (got, ref, floor))):
+                check(nm, a, r, f)
+        else:
+            check(k, got[k], ref[k], floor[k])
+    assert not bad, bad
