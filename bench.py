@@ -232,7 +232,9 @@ def bench_core(steps, warmup):
         for t in leaves:
             t.grad = None
         out = mamba2_fused_kernel_with_caching(zx, A, D, cw, cb, dtb, nw, g, n, d, p)
-        out.backward(dout)
+        # the core computes and returns d_zxBCdt as always; autograd is only told not to copy it into zx.grad (in the layer
+        # zxBCdt is the projection's output and its gradient goes straight into that GEMM's backward, no copy either)
+        out.backward(dout, inputs=leaves[1:])
 
     wall_ms, per = event_time_ms(step, steps, warmup)
     ms = sum(per) / len(per)

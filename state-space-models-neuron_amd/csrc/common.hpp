@@ -165,6 +165,16 @@ __device__ __forceinline__ float warp_sum(float v) {
     return v;
 }
 
+// Number of compute units of the current device (queried once per process; 256 on MI355X).
+inline int64_t device_cus() {
+    static int64_t cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        return (int64_t)n;
+    }();
+    return cus;
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }

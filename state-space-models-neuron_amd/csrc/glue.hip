@@ -132,26 +132,29 @@ __device__ __forceinline__ void store_vec(T* p, const float (&v)[GlueVec<T>::V])
 // sum over the WPG waves that share a (row, group); `slot` alternates between two LDS rows so that one barrier per
 // reduction is enough
 template <int WPG>
-__device__ __forceinline__ void group_sum2(float& a, float& b, float (*red)[2][4], int slot) {
+__device__ __forceinline__ void group_sum2(float& a, float& b, float (*red)[2][8], int slot) {
     a = warp_sum(a); b = warp_sum(b);
-    if constexpr (WPG == 4) {
+    if constexpr (WPG > 1) {
         const int wave = threadIdx.x >> 6;
         if ((threadIdx.x & 63) == 0) { red[slot][0][wave] = a; red[slot][1][wave] = b; }
         __syncthreads();
-        a = (red[slot][0][0] + red[slot][0][1]) + (red[slot][0][2] + red[slot][0][3]);
-        b = (red[slot][1][0] + red[slot][1][1]) + (red[slot][1][2] + red[slot][1][3]);
+        a = red[slot][0][0]; b = red[slot][1][0];
+#pragma unroll
+        for (int q = 1; q < WPG; ++q) { a += red[slot][0][q]; b += red[slot][1][q]; }      // fixed order
     }
 }
 
-// grid (row blocks, groups), 256 threads.  WPG = waves per (row, group): 1 or 4.  NV = vectors per lane.
-template <typename T, int WPG, int NV, bool BWD>
-__global__ void __launch_bounds__(256)
+// grid (row blocks, groups).  WPG = waves per (row, group): 1 (256 threads, each wave its own rows) or 4 or 5 (the whole
+// workgroup of WPG waves shares a row).  NV = vectors per lane.  GATED: z given.  EXACT: the group is exactly WPG x 64 x NV
+// vectors wide, so no lane is idle and nothing is masked (5120 channels of a 16-bit type = 5 waves x 2 vectors).
+template <typename T, int WPG, int NV, bool BWD, bool GATED, bool EXACT>
+__global__ void __launch_bounds__(WPG == 1 ? 256 : WPG * 64)
 rmsnorm_gated_kernel(const NormArgs a) {
     constexpr int V = GlueVec<T>::V;
     constexpr int TPG = WPG * 64;                 // threads per (row, group)
-    __shared__ float red[2][2][4];
+    __shared__ float red[2][2][8];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int tl = WPG == 4 ? tid : lane;         // index inside the (row, group)
+    const int tl = WPG > 1 ? tid : lane;          // index inside the (row, group)
     const int64_t grp = blockIdx.y;
     const int64_t c0 = grp * a.gw;                // first channel of the group
     const int nvec = (int)(a.gw / V);
@@ -163,35 +166,38 @@ rmsnorm_gated_kernel(const NormArgs a) {
         const int vi = it * TPG + tl;
 #pragma unroll
         for (int e = 0; e < V; ++e) {
-            w[it][e] = vi < nvec ? a.w[c0 + (int64_t)vi * V + e] : 0.f;
+            w[it][e] = (EXACT || vi < nvec) ? a.w[c0 + (int64_t)vi * V + e] : 0.f;
             if (BWD) dw[it][e] = 0.f;
         }
     }
-    const int64_t r0 = (int64_t)blockIdx.x * a.rows_per_block;
-    const int64_t r1 = r0 + a.rows_per_block < a.rows ? r0 + a.rows_per_block : a.rows;
+    // Rows are dealt out round-robin: workgroup i (WPG > 1; wave 4 i + w for WPG == 1) takes rows i, i + G, i + 2 G, ... with G
+    // the number of workgroups (waves), so that at any moment the rows in flight over the whole chip are neighbours in
+    // memory and every memory channel is in use.  (A contiguous block of rows per workgroup puts all workgroups a fixed
+    // power-of-two-rich distance apart, and they then walk through the same channels together: 3.6 TB/s for the loads alone.)
+    const int64_t r1 = a.rows;
+    const int64_t RSTEP = WPG > 1 ? (int64_t)gridDim.x : (int64_t)gridDim.x * 4;
     int slot = 0;
-    // WPG == 4: every wave takes every row of the block (uniform trip count, barriers inside); WPG == 1: wave w takes rows w, w + 4, ...
-    // the raw vectors of the next row are loaded before this row is reduced (the row after the last: the last once more)
-    constexpr int RSTEP = WPG == 4 ? 1 : 4;
-    const bool gated = a.z != nullptr;
+    // WPG > 1: every wave takes every row of the workgroup (uniform trip count, barriers inside); WPG == 1: each wave its own rows.
+    // the raw vectors of the next row are loaded before this row is reduced (the row after the last: the first once more)
+    constexpr bool gated = GATED;
     // the forward keeps two register sets and loads a row a whole iteration before it is used (the backward has no
     // registers left for that: it loads the next row behind the first pass over the current one)
     uint4 rxa[NV], rza[NV], rxb[BWD ? 1 : NV], rzb[BWD ? 1 : NV], rg[BWD ? NV : 1];
+    const int64_t rfirst = WPG > 1 ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + wave;
     auto load_row = [&](int64_t r, uint4 (&rx)[NV], uint4 (&rz)[NV]) {
-        const int64_t rr = r < r1 ? r : r1 - 1;
+        const int64_t rr = r < r1 ? r : rfirst;
         const T* xr = static_cast<const T*>(a.x) + rr * a.x_sr + c0;
         const T* zr = gated ? static_cast<const T*>(a.z) + rr * a.z_sr + c0 : xr;
         const T* gr = BWD ? static_cast<const T*>(a.g) + rr * a.g_sr + c0 : xr;
 #pragma unroll
         for (int it = 0; it < NV; ++it) {
             const int vi = it * TPG + tl;
-            const int64_t off = (int64_t)(vi < nvec ? vi : 0) * V;      // idle lanes read the first vector and ignore it
+            const int64_t off = (int64_t)((EXACT || vi < nvec) ? vi : 0) * V;      // idle lanes read the first vector and ignore it
             rx[it] = *reinterpret_cast<const uint4*>(xr + off);
-            rz[it] = *reinterpret_cast<const uint4*>(zr + off);
+            if (gated) rz[it] = *reinterpret_cast<const uint4*>(zr + off);
             if (BWD) rg[it] = *reinterpret_cast<const uint4*>(gr + off);
         }
     };
-    const int64_t rfirst = r0 + (WPG == 4 ? 0 : wave);
     if (rfirst < r1) load_row(rfirst, rxa, rza);
     auto do_row = [&](int64_t r, uint4 (&rx)[NV], uint4 (&rz)[NV]) {
         const bool zr = gated;
@@ -201,12 +207,14 @@ rmsnorm_gated_kernel(const NormArgs a) {
         for (int it = 0; it < NV; ++it) {
             const int vi = it * TPG + tl;
             float xv[V], zv[V], gv[V];
-            unpack_vec<T>(rx[it], xv);
-            unpack_vec<T>(rz[it], zv);
+            // an idle lane's x is zeroed as a raw vector (four selects): h, and with it every sum, is then zero there
+            uint4 rxv = rx[it];
+            if (!EXACT && vi >= nvec) rxv = uint4{0u, 0u, 0u, 0u};
+            unpack_vec<T>(rxv, xv);
+            if (gated) unpack_vec<T>(rz[it], zv);
             if (BWD) unpack_vec<T>(rg[it], gv);
 #pragma unroll
             for (int e = 0; e < V; ++e) {
-                if (vi >= nvec) { xv[e] = 0.f; zv[e] = 0.f; if (BWD) gv[e] = 0.f; }
                 const float gate = zr ? silu_f(zv[e]) : 1.f;
                 h[it][e] = xv[e] * gate;
                 ss += h[it][e] * h[it][e];
@@ -225,7 +233,7 @@ rmsnorm_gated_kernel(const NormArgs a) {
 #pragma unroll
             for (int it = 0; it < NV; ++it) {
                 const int vi = it * TPG + tl;
-                if (vi >= nvec) continue;
+                if (!EXACT && vi >= nvec) continue;
                 float o[V];
 #pragma unroll
                 for (int e = 0; e < V; ++e) o[e] = w[it][e] * (h[it][e] * rinv);
@@ -242,16 +250,20 @@ rmsnorm_gated_kernel(const NormArgs a) {
 #pragma unroll
             for (int it = 0; it < NV; ++it) {
                 const int vi = it * TPG + tl;
-                if (vi >= nvec) continue;
+                if (!EXACT && vi >= nvec) continue;
                 float ox[V], oz[V];
 #pragma unroll
                 for (int e = 0; e < V; ++e) {
                     const float gwv = gs[it][e] * w[it][e];
                     const float dh = rinv * (gwv - cf * h[it][e]);
-                    const float z = zs[it][e];
-                    const float s = sigmoid_f(z);
-                    ox[e] = dh * (zr ? z * s : 1.f);
-                    oz[e] = dh * xs[it][e] * (s * (1.f + z * (1.f - s)));
+                    if (zr) {
+                        const float z = zs[it][e];
+                        const float s = sigmoid_f(z);
+                        ox[e] = dh * (z * s);
+                        oz[e] = dh * xs[it][e] * (s * (1.f + z * (1.f - s)));
+                    } else {
+                        ox[e] = dh; oz[e] = 0.f;
+                    }
                     dw[it][e] += gs[it][e] * (h[it][e] * rinv);
                 }
                 store_vec<T>(static_cast<T*>(a.dx) + r * a.dx_sr + c0 + (int64_t)vi * V, ox);
@@ -266,20 +278,20 @@ rmsnorm_gated_kernel(const NormArgs a) {
         for (int64_t r = rfirst; r < r1; r += 2 * RSTEP) {
             load_row(r + RSTEP, rxb, rzb);
             do_row(r, rxa, rza);
-            if (r + RSTEP < r1) {      // uniform over the workgroup when it shares its rows (WPG == 4)
+            if (r + RSTEP < r1) {      // uniform over the workgroup when it shares its rows (WPG > 1)
                 load_row(r + 2 * RSTEP, rxa, rza);
                 do_row(r + RSTEP, rxb, rzb);
             }
         }
     }
     if (BWD) {
-        // one partial row per workgroup (WPG == 4: each lane owns its channels) or per wave (WPG == 1)
-        const int64_t prow = WPG == 4 ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + wave;
+        // one partial row per workgroup (WPG > 1: each lane owns its channels) or per wave (WPG == 1)
+        const int64_t prow = WPG > 1 ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + wave;
         float* pp = a.partial + prow * a.d + c0;
 #pragma unroll
         for (int it = 0; it < NV; ++it) {
             const int vi = it * TPG + tl;
-            if (vi >= nvec) continue;
+            if (!EXACT && vi >= nvec) continue;
 #pragma unroll
             for (int q = 0; q < V / 4; ++q)
                 *reinterpret_cast<floatx4*>(pp + (int64_t)vi * V + 4 * q) = floatx4{dw[it][4 * q], dw[it][4 * q + 1], dw[it][4 * q + 2], dw[it][4 * q + 3]};
@@ -294,15 +306,22 @@ int64_t norm_rows_per_block(int64_t rows, int64_t groups, bool bwd) {
     if (rb < 4) rb = 4;
     return (rb + 3) / 4 * 4;
 }
-// the forward with four waves per (row, group) takes one row per pass: few rows (a decode step) spread over more workgroups
+// The forward with a whole workgroup per (row, group): few rows (a decode step) are spread one per workgroup; many rows go
+// to exactly ONE workgroup per compute unit (measured at 8192 rows of 5120 channels, rows dealt round-robin: 256 workgroups
+// 46 us, 192 -> 55, 320 -> 57, 512 -> 52, 1024 -> 54: more resident waves only disturb the three streams).
 int64_t norm_rows_per_block_fwd(int64_t rows, int64_t groups, int64_t nvec) {
-    if (nvec > 256 && rows * groups < 4096) return 1;
+    if (nvec > 256) {
+        if (rows * groups < 4096) return 1;
+        return ceil_div(rows * groups, device_cus());
+    }
     return norm_rows_per_block(rows, groups, false);
 }
 // waves per (row, group) and vectors per lane for a group of `nvec` 16-byte vectors; false if it does not fit
 bool norm_shape(int64_t nvec, int vec_elems, int* wpg, int* nv) {
     if (nvec <= 0) return false;
     if (nvec <= 256) { *wpg = 1; *nv = (int)((nvec + 63) / 64); return true; }
+    // a group that five waves cover with no idle lane (5120 channels: the 2.7B width) takes five
+    if (nvec % 320 == 0 && (nvec / 320 == 2 || nvec / 320 == 4) && nvec * vec_elems <= 8192) { *wpg = 5; *nv = (int)(nvec / 320); return true; }
     // up to 8192 channels per group in either type: 4 vectors of 8 per lane (16-bit), 8 vectors of 4 (fp32)
     if (nvec * vec_elems <= 8192) { *wpg = 4; *nv = (int)((nvec + 255) / 256); return true; }
     return false;
@@ -315,11 +334,17 @@ int launch_norm(const NormArgs& a, int64_t groups, hipStream_t st) {
     if (!norm_shape(a.gw / V, V, &wpg, &nv))
         return fail(M2_ERR_SHAPE, "rmsnorm_gated: %lld channels per group exceed the supported 8192", (long long)a.gw);
     const dim3 grid((unsigned)ceil_div(a.rows, a.rows_per_block), (unsigned)groups);
-#define M2_NORM_CASE(W, N) if (wpg == W && nv == N) { rmsnorm_gated_kernel<T, W, N, BWD><<<grid, 256, 0, st>>>(a); return check_launch("rmsnorm_gated_kernel"); }
+    const bool exact = (int64_t)wpg * 64 * nv == a.gw / V, gated = a.z != nullptr;
+#define M2_NORM_LAUNCH(W, N, G, E) { rmsnorm_gated_kernel<T, W, N, BWD, G, E><<<grid, (W == 1 ? 256 : W * 64), 0, st>>>(a); return check_launch("rmsnorm_gated_kernel"); }
+#define M2_NORM_CASE(W, N) if (wpg == W && nv == N) { \
+        if (gated) { if (exact) M2_NORM_LAUNCH(W, N, true, true) else M2_NORM_LAUNCH(W, N, true, false) } \
+        else { if (exact) M2_NORM_LAUNCH(W, N, false, true) else M2_NORM_LAUNCH(W, N, false, false) } }
     M2_NORM_CASE(1, 1) M2_NORM_CASE(1, 2) M2_NORM_CASE(1, 3) M2_NORM_CASE(1, 4)
     M2_NORM_CASE(4, 2) M2_NORM_CASE(4, 3) M2_NORM_CASE(4, 4)
+    M2_NORM_CASE(5, 2) M2_NORM_CASE(5, 4)
     if constexpr (sizeof(T) == 4) { M2_NORM_CASE(4, 5) M2_NORM_CASE(4, 6) M2_NORM_CASE(4, 7) M2_NORM_CASE(4, 8) }
 #undef M2_NORM_CASE
+#undef M2_NORM_LAUNCH
     return fail(M2_ERR_SHAPE, "rmsnorm_gated: no kernel for %d waves x %d vectors", wpg, nv);
 }
 
@@ -493,7 +518,7 @@ extern "C" int m2_rmsnorm_gated_bwd(const m2_rmsnorm_params* p, void* stream) {
         int wpg = 0, nv = 0;
         if (!norm_shape(a.gw / V, V, &wpg, &nv))
             return fail(M2_ERR_SHAPE, "rmsnorm_gated_bwd: %lld channels per group exceed the supported 8192", (long long)a.gw);
-        prows = ceil_div(p->rows, a.rows_per_block) * (wpg == 4 ? 1 : 4);
+        prows = ceil_div(p->rows, a.rows_per_block) * (wpg > 1 ? 1 : 4);
         M2_DISPATCH_DTYPE(p->dtype, T, rc = (launch_norm<T, true>(a, p->n_groups, st)));
         if (rc) return rc;
     }

@@ -26,16 +26,6 @@ struct SsdWorkspace {
     size_t kept_bytes = 0;              // size of the forward -> backward carry-over (chunk_states buffer)
 };
 
-// Number of compute units of the current device (queried once per process; 256 on MI355X).
-inline int64_t device_cus() {
-    static int64_t cus = [] {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        return (int64_t)n;
-    }();
-    return cus;
-}
-
 // A workgroup owns one chunk of one group and loops over a slice of that group's heads (operands shared by the
 // group stay on chip, group-level reductions happen in registers).  The slice count is the smallest divisor of
 // heads-per-group that gives at least `wgs_per_cu` workgroups per compute unit: the grid then fills the GPU in one

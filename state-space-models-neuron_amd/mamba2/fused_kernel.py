@@ -41,6 +41,20 @@ def _views(zxBCdt, n_groups, d_state, d_inner, d_head):
     return z, xBC, dt, h, d_conv
 
 
+def _empty_rows_128(like):
+    """An uninitialised (b, l, width) tensor like ``like`` whose row pitch is a whole number of 128-byte cache lines (the
+    width itself when it already is one: 18560 columns of the 7B layer; 10576 columns of bf16 are 165.25 lines, and every
+    wave-wide access to a column slice of such a buffer straddles two lines in three rows out of four).  The padded form is
+    a column slice of a wider allocation: consumers that take a leading dimension (the projection's backward GEMM) read
+    it in place."""
+    b, l, width = like.shape
+    per_line = 128 // like.element_size()
+    pitch = -(-width // per_line) * per_line
+    if pitch == width:
+        return torch.empty((b, l, width), dtype=like.dtype, device=like.device)
+    return torch.empty((b, l, pitch), dtype=like.dtype, device=like.device)[..., :width]
+
+
 def _xbc_views(conv_out, n_groups, d_state, d_inner, d_head):
     h = d_inner // d_head
     gn = n_groups * d_state
@@ -69,7 +83,7 @@ def _backward_parts(d_output, zxBCdt, logA, D, conv_w, conv_b, dt_bias, norm_w, 
                     n_groups, d_state, d_inner, d_head):
     z, xBC, dt, h, d_conv = _views(zxBCdt, n_groups, d_state, d_inner, d_head)
     b, l, width = zxBCdt.shape
-    d_zxBCdt = torch.empty_like(zxBCdt, memory_format=torch.contiguous_format)
+    d_zxBCdt = _empty_rows_128(zxBCdt)
     dz_view = d_zxBCdt[..., :d_inner]
     dxBC_view = d_zxBCdt[..., d_inner:d_inner + d_conv]
     ddt_view = d_zxBCdt[..., d_inner + d_conv:]
