@@ -180,11 +180,15 @@ rmsnorm_gated_kernel(const NormArgs a) {
     // WPG > 1: every wave takes every row of the workgroup (uniform trip count, barriers inside); WPG == 1: each wave its own rows.
     // the raw vectors of the next row are loaded before this row is reduced (the row after the last: the first once more)
     constexpr bool gated = GATED;
-    // the forward keeps two register sets and loads a row a whole iteration before it is used (the backward has no
-    // registers left for that: it loads the next row behind the first pass over the current one)
-    uint4 rxa[NV], rza[NV], rxb[BWD ? 1 : NV], rzb[BWD ? 1 : NV], rg[BWD ? NV : 1];
+    // Two register sets, a row loaded a whole iteration before it is used: the forward always; the backward where the
+    // workgroup is alone on its compute unit anyway (five waves: up to 256 registers each).  Otherwise the backward loads
+    // the next row behind the first pass over the current one.
+    constexpr bool TWO = !BWD || WPG == 5;
+    struct RowRegs { uint4 x[NV], z[NV], g[BWD ? NV : 1]; };
+    RowRegs ra, rb;
     const int64_t rfirst = WPG > 1 ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + wave;
-    auto load_row = [&](int64_t r, uint4 (&rx)[NV], uint4 (&rz)[NV]) {
+    auto load_row = [&](int64_t r, RowRegs& q) {
+        uint4 (&rx)[NV] = q.x; uint4 (&rz)[NV] = q.z; uint4 (&rg)[BWD ? NV : 1] = q.g;
         const int64_t rr = r < r1 ? r : rfirst;
         const T* xr = static_cast<const T*>(a.x) + rr * a.x_sr + c0;
         const T* zr = gated ? static_cast<const T*>(a.z) + rr * a.z_sr + c0 : xr;
@@ -198,8 +202,9 @@ rmsnorm_gated_kernel(const NormArgs a) {
             if (BWD) rg[it] = *reinterpret_cast<const uint4*>(gr + off);
         }
     };
-    if (rfirst < r1) load_row(rfirst, rxa, rza);
-    auto do_row = [&](int64_t r, uint4 (&rx)[NV], uint4 (&rz)[NV]) {
+    if (rfirst < r1) load_row(rfirst, ra);
+    auto do_row = [&](int64_t r, RowRegs& q) {
+        uint4 (&rx)[NV] = q.x; uint4 (&rz)[NV] = q.z; uint4 (&rg)[BWD ? NV : 1] = q.g;
         const bool zr = gated;
         float h[NV][V], xs[BWD ? NV : 1][V], zs[BWD ? NV : 1][V], gs[BWD ? NV : 1][V];
         float ss = 0.f, dot = 0.f;
@@ -224,7 +229,7 @@ rmsnorm_gated_kernel(const NormArgs a) {
                 }
             }
         }
-        if (BWD) load_row(r + RSTEP, rx, rz);
+        if (!TWO) load_row(r + RSTEP, q);
         group_sum2<WPG>(ss, dot, red, slot);
         slot ^= 1;
         const float var = ss * inv_n + a.eps;
@@ -271,16 +276,16 @@ rmsnorm_gated_kernel(const NormArgs a) {
             }
         }
     };
-    if constexpr (BWD) {
-        for (int64_t r = rfirst; r < r1; r += RSTEP) do_row(r, rxa, rza);
+    if constexpr (!TWO) {
+        for (int64_t r = rfirst; r < r1; r += RSTEP) do_row(r, ra);
     } else {
         // rows in pairs, one per register set; a row's loads are issued before the row in front of it is processed
         for (int64_t r = rfirst; r < r1; r += 2 * RSTEP) {
-            load_row(r + RSTEP, rxb, rzb);
-            do_row(r, rxa, rza);
+            load_row(r + RSTEP, rb);
+            do_row(r, ra);
             if (r + RSTEP < r1) {      // uniform over the workgroup when it shares its rows (WPG > 1)
-                load_row(r + 2 * RSTEP, rxa, rza);
-                do_row(r + RSTEP, rxb, rzb);
+                load_row(r + 2 * RSTEP, ra);
+                do_row(r + RSTEP, rb);
             }
         }
     }
@@ -305,6 +310,12 @@ int64_t norm_rows_per_block(int64_t rows, int64_t groups, bool bwd) {
     int64_t rb = rows * groups / (bwd ? 512 : 1024);
     if (rb < 4) rb = 4;
     return (rb + 3) / 4 * 4;
+}
+// The backward with a whole workgroup per (row, group): one workgroup per compute unit as well (it is alone there by its
+// register count anyway; 256 workgroups 77 us, 512 -> 80, 768 -> 95 at 8192 rows of 5120 channels).
+int64_t norm_rows_per_block_bwd(int64_t rows, int64_t groups, int64_t nvec) {
+    if (nvec > 256 && rows * groups >= 4096) return ceil_div(rows * groups, device_cus());
+    return norm_rows_per_block(rows, groups, true);
 }
 // The forward with a whole workgroup per (row, group): few rows (a decode step) are spread one per workgroup; many rows go
 // to exactly ONE workgroup per compute unit (measured at 8192 rows of 5120 channels, rows dealt round-robin: 256 workgroups
@@ -486,7 +497,8 @@ extern "C" int m2_rmsnorm_gated_fwd(const m2_rmsnorm_params* p, void* stream) {
 
 extern "C" size_t m2_rmsnorm_gated_bwd_workspace_bytes(int64_t rows, int64_t channels, int32_t n_groups, int32_t dtype) {
     if (rows <= 0 || channels <= 0 || n_groups <= 0) return 256;
-    const int64_t nrb = m2::ceil_div(rows, m2::norm_rows_per_block(rows, n_groups, true));
+    const int64_t nvec = channels / n_groups / (dtype == M2_F32 ? 4 : 8);
+    const int64_t nrb = m2::ceil_div(rows, m2::norm_rows_per_block_bwd(rows, n_groups, nvec));
     return m2::align_up((size_t)nrb * 4 * (size_t)channels * sizeof(float), 256);      // up to one partial row per wave
 }
 
@@ -514,7 +526,7 @@ extern "C" int m2_rmsnorm_gated_bwd(const m2_rmsnorm_params* p, void* stream) {
         a.g = p->d_out; a.g_sr = p->d_out_stride_row; a.dx = p->dx; a.dx_sr = p->dx_stride_row; a.dz = p->dz; a.dz_sr = p->dz_stride_row;
         a.partial = static_cast<float*>(p->workspace);
         a.rows = p->rows; a.d = p->channels; a.gw = p->channels / p->n_groups; a.eps = p->eps;
-        a.rows_per_block = norm_rows_per_block(p->rows, p->n_groups, true);
+        a.rows_per_block = norm_rows_per_block_bwd(p->rows, p->n_groups, a.gw / V);
         int wpg = 0, nv = 0;
         if (!norm_shape(a.gw / V, V, &wpg, &nv))
             return fail(M2_ERR_SHAPE, "rmsnorm_gated_bwd: %lld channels per group exceed the supported 8192", (long long)a.gw);

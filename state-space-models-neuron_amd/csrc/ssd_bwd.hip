@@ -613,15 +613,16 @@ int ssd_bwd_impl(const m2_ssd_params* p, hipStream_t st) {
     // gradient of the state leaving each chunk (reverse recurrence over the chunks' own contributions)
     if constexpr (sizeof(T) == 2) {
         // the main backward kernel forms dlam itself when it runs; otherwise this pass does (and reads the forward states for it)
-        auto k = state_pass16_kernel<T, P, N, true, !bwd16_ok<T, P, N>()>;
-        const size_t sm = state_pass_smem<P, N>();
+        constexpr int SPLIT = kStatePassSplit;
+        auto k = state_pass16_kernel<T, P, N, true, !bwd16_ok<T, P, N>(), false, SPLIT>;
+        const size_t sm = state_pass_smem<P, N, false, SPLIT>();
         if ((rc = allow_smem(k, sm))) return rc;
         StatePassArgs sa;
         sa.X = dy; sa.X_sb = p->dy_stride_b; sa.X_sl = p->dy_stride_l; sa.X_sh = p->dy_stride_h;
         sa.ldtab = w.ldtab; sa.Mt = w.Ct; sa.init = p->d_final_state; sa.prev = w.dprev; sa.final_out = p->d_initial_state;
         sa.sprev = w.prev; sa.dlam = w.dlam;
         sa.seqlen = p->seqlen; sa.nheads = p->nheads; sa.ngroups = p->ngroups; sa.nchunks = nc;
-        k<<<dim3((unsigned)(p->nheads * kStatePassSplit), (unsigned)p->batch), state_pass_threads<N>(), sm, st>>>(sa);
+        k<<<dim3((unsigned)(p->nheads * SPLIT), (unsigned)p->batch), state_pass_threads<N>(), sm, st>>>(sa);
         if ((rc = check_launch("ssd state_pass16_kernel<reverse>"))) return rc;
     } else
     {   // fp32: local dS contributions (reuses the `local` region), then the reverse recurrence

@@ -189,15 +189,16 @@ inline int ssd_launch_states(const m2_ssd_params* p, const SsdWorkspace& w, floa
         // (3.7 us more per pass at b4 l2048 h80; the states entering the chunks come out of the same accumulators, so y
         // differs from the one-tile form in the last bit here and there)
         const bool hilo = final_out != nullptr;
-        auto k = hilo ? state_pass16_kernel<T, P, N, false, false, true> : state_pass16_kernel<T, P, N, false>;
-        const size_t sm = hilo ? state_pass_smem<P, N, true>() : state_pass_smem<P, N>();
+        constexpr int SPLIT = kStatePassSplit;
+        auto k = hilo ? state_pass16_kernel<T, P, N, false, false, true, SPLIT> : state_pass16_kernel<T, P, N, false, false, false, SPLIT>;
+        const size_t sm = hilo ? state_pass_smem<P, N, true, SPLIT>() : state_pass_smem<P, N, false, SPLIT>();
         if ((rc = allow_smem(k, sm))) return rc;
         StatePassArgs sa;
         sa.X = x; sa.X_sb = p->x_stride_b; sa.X_sl = p->x_stride_l; sa.X_sh = p->x_stride_h;
         sa.ldtab = w.ldtab; sa.Mt = w.Bt; sa.init = p->initial_state; sa.prev = w.prev; sa.final_out = final_out;
         sa.sprev = nullptr; sa.dlam = nullptr;
         sa.seqlen = p->seqlen; sa.nheads = p->nheads; sa.ngroups = p->ngroups; sa.nchunks = nc;
-        k<<<dim3((unsigned)(p->nheads * kStatePassSplit), (unsigned)p->batch), state_pass_threads<N>(), sm, st>>>(sa);
+        k<<<dim3((unsigned)(p->nheads * SPLIT), (unsigned)p->batch), state_pass_threads<N>(), sm, st>>>(sa);
         return check_launch("ssd state_pass16_kernel");
     } else {
         // fp32 operands: per-chunk contributions (fp32, workspace), then the recurrence over the chunks

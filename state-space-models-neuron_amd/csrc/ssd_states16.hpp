@@ -38,26 +38,28 @@ struct StatePassArgs {
 };
 
 // workgroups per (batch, head): each takes half of the state rows (more, smaller workgroups: the chunk loop is a chain of
-// dependent memory round trips, and only other resident waves can fill its gaps)
+// dependent memory round trips, and only other resident waves can fill its gaps).  One workgroup per head (SPLIT = 1: whole
+// 128-byte x rows, each operand fragment feeding two products, half the fragment traffic) is slower: reverse pass 52 -> 57 us,
+// forward pass with the two-tile operands 56 -> 79 us at b4 l2048 h80.
 constexpr int kStatePassSplit = 2;
 // one wave per 32 state columns
 template <int N> constexpr int state_pass_threads() { return (N / 32) * 64; }
-template <int P, int N, bool HILO = false>
+template <int P, int N, bool HILO = false, int SPLIT = kStatePassSplit>
 constexpr size_t state_pass_smem() {
-    return (size_t)(HILO ? 2 : 1) * 2 * kQ * (P / 2) * 2 + (size_t)2 * (P / 2) * (N + 8) * 2;
+    return (size_t)(HILO ? 2 : 1) * 2 * kQ * (P / SPLIT) * 2 + (size_t)2 * (P / SPLIT) * (N + 8) * 2;
 }
 
 // HILO: the scaled rows are staged as TWO 16-bit tiles, the rounded value and the rounded remainder, and each k step takes
 // two products, so that the fp32 scale dt e^{Lam - l} reaches the accumulators with 16 significand bits instead of 8 (the
 // final state is an fp32 output; with one tile its error is that of the operand rounding, 2^-9 of every term).
-template <typename T, int P, int N, bool REVERSE, bool DLAM = REVERSE, bool HILO = false>
-__global__ void __launch_bounds__(state_pass_threads<N>(), (P == 64 ? (DLAM ? 2 : 3) : (DLAM ? 1 : 2)))
+template <typename T, int P, int N, bool REVERSE, bool DLAM = REVERSE, bool HILO = false, int SPLIT = kStatePassSplit>
+__global__ void __launch_bounds__(state_pass_threads<N>(), (SPLIT == 1 ? (P == 64 ? 2 : 1) : (P == 64 ? (DLAM ? 2 : 3) : (DLAM ? 1 : 2))))
 state_pass16_kernel(const StatePassArgs a) {
     static_assert(sizeof(T) == 2, "16-bit operands only");
     constexpr int NWAVES = N / 32, THREADS = state_pass_threads<N>();
-    constexpr int PH = P / 2;                          // state rows (head channels) of this workgroup
+    constexpr int PH = P / SPLIT;                      // state rows (head channels) of this workgroup
     constexpr int NW = 32;                             // state columns per wave
-    static_assert(kStatePassSplit * NWAVES <= kDlamParts, "dlam slots");
+    static_assert(SPLIT * NWAVES <= kDlamParts, "dlam slots");
     constexpr int PBW = PH / 32, NBW = 1;              // 32x32 blocks per wave
     constexpr int SPR_X = PH / 8;                      // 16-byte slots per staged x row
     constexpr int NXR = kQ * SPR_X / THREADS;              // x pieces per thread per chunk
@@ -95,7 +97,7 @@ state_pass16_kernel(const StatePassArgs a) {
         for (int j = 0; j < NBW; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int row = pw * (P / 2) + i * 32 + r, col = n0 + j * 32 + acc_row(lane, v);
+                const int row = pw * PH + i * 32 + r, col = n0 + j * 32 + acc_row(lane, v);
                 acc[i][j][v] = a.init ? a.init[bh * (P * N) + row * N + col] : 0.f;
             }
 
@@ -234,8 +236,7 @@ state_pass16_kernel(const StatePassArgs a) {
             if (lane == 0) {
                 const int slot = pw * NWAVES + wave;
                 a.dlam[(bh * nc + c) * kDlamParts + slot] = dec * dot;
-                if (kStatePassSplit * NWAVES < kDlamParts && slot + kStatePassSplit * NWAVES < kDlamParts)
-                    a.dlam[(bh * nc + c) * kDlamParts + slot + kStatePassSplit * NWAVES] = 0.f;
+                for (int s2 = slot + SPLIT * NWAVES; s2 < kDlamParts; s2 += SPLIT * NWAVES) a.dlam[(bh * nc + c) * kDlamParts + s2] = 0.f;
             }
         }
 
@@ -302,7 +303,7 @@ state_pass16_kernel(const StatePassArgs a) {
             for (int j = 0; j < NBW; ++j)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const int row = pw * (P / 2) + i * 32 + r, col = n0 + j * 32 + acc_row(lane, v);
+                    const int row = pw * PH + i * 32 + r, col = n0 + j * 32 + acc_row(lane, v);
                     a.final_out[bh * (P * N) + row * N + col] = acc[i][j][v];
                 }
     }
