@@ -132,7 +132,7 @@ __device__ __forceinline__ void store_vec(T* p, const float (&v)[GlueVec<T>::V])
 // sum over the WPG waves that share a (row, group); `slot` alternates between two LDS rows so that one barrier per
 // reduction is enough
 template <int WPG>
-__device__ __forceinline__ void group_sum2(float& a, float& b, float (*red)[2][8], int slot) {
+__device__ __forceinline__ void group_sum2(float& a, float& b, float (*red)[2][16], int slot) {
     a = warp_sum(a); b = warp_sum(b);
     if constexpr (WPG > 1) {
         const int wave = threadIdx.x >> 6;
@@ -152,7 +152,7 @@ __global__ void __launch_bounds__(WPG == 1 ? 256 : WPG * 64)
 rmsnorm_gated_kernel(const NormArgs a) {
     constexpr int V = GlueVec<T>::V;
     constexpr int TPG = WPG * 64;                 // threads per (row, group)
-    __shared__ float red[2][2][8];
+    __shared__ float red[2][2][16];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int tl = WPG > 1 ? tid : lane;          // index inside the (row, group)
     const int64_t grp = blockIdx.y;
