@@ -29,10 +29,10 @@ HBM_PEAK_GBS = 8000.0              # MI355X HBM3E
 # HBM bytes per step as PROFILED (two rocprofv3 --pmc runs of this file, FETCH_SIZE then WRITE_SIZE, each scaled by what
 # the same counter reads for the 1 GiB copy kernel in the same run; summaries under profiles/).  They are constants of
 # the kernels as last profiled, not measurements of this run: `traffic_source` in the JSON says so.
-SSD_TRAFFIC_BYTES = 1.449e9
+SSD_TRAFFIC_BYTES = 1.460e9
 CONV_TRAFFIC_BYTES = 489.3e6
-DECODE_TRAFFIC_BYTES = 64 * 689.3e6
-GLUE_TRAFFIC_BYTES = 703.5e6
+DECODE_TRAFFIC_BYTES = 64 * 689.2e6
+GLUE_TRAFFIC_BYTES = 710.5e6
 TRAFFIC_SOURCE = "profiled constant: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this workload, scaled by the 1 GiB copy kernel; not measured in this run"
 
 SSD_CFG = dict(b=4, l=2048, h=80, p=64, n=128, g=1)
