@@ -466,6 +466,58 @@ def bench_copy(steps, warmup):
                           "kernels": "stream_copy_kernel"})
 
 
+def bench_access_pattern(steps, warmup):
+    """What the memory system gives a kernel with the SSD kernels' streams and no arithmetic: x of the c1 shape (b4 l2048,
+    80 heads of 128 bytes per token row) read as per-head tiles of 128 rows and written back as contiguous tiles, against
+    a plain copy of the same 84 MB.  A 1 GiB read in front of every timed launch leaves the caches holding none of it."""
+    import torch
+    from mamba2 import _lib
+    lib = _lib.load()
+    batch, rows, row_bytes = SSD_CFG["b"], SSD_CFG["l"], SSD_CFG["h"] * SSD_CFG["p"] * 2
+    g = torch.Generator().manual_seed(0)
+    src = torch.randint(0, 256, (batch * rows * row_bytes,), generator=g, dtype=torch.uint8).to("cuda:0")
+    dst = torch.empty_like(src)
+    sweep = torch.ones(1 << 28, dtype=torch.int32, device="cuda:0")
+    stream = lambda: torch.cuda.current_stream().cuda_stream
+
+    def timed(launch):
+        for _ in range(max(2, warmup // 2)):
+            launch()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(max(5, steps // 2))]
+        for s, e in evs:
+            sweep.sum()
+            s.record()
+            rc = launch()
+            e.record()
+            if rc != 0:
+                raise RuntimeError(lib.m2_last_error().decode())
+        torch.cuda.synchronize()
+        t = sorted(s.elapsed_time(e) for s, e in evs)
+        return t[len(t) // 2]
+
+    moved = 2 * src.numel()
+    rows_out = []
+    cases = [("plain copy (stream_copy_kernel)", lambda: lib.m2_stream_copy(src.data_ptr(), dst.data_ptr(), src.numel(), stream()))]
+    for piece, in_order, what in ((64, 1, "half-head tiles in chunk order, one workgroup per (batch, half head): the state passes' streams"),
+                                  (128, 1, "whole-head tiles in chunk order, one workgroup per (batch, head)"),
+                                  (128, 0, "whole-head tiles, one workgroup per tile: the chunk-parallel kernels' streams"),
+                                  (256, 0, "two-head tiles, one workgroup per tile"),
+                                  (512, 0, "four-head tiles, one workgroup per tile")):
+        cases.append((f"{what} ({piece}-byte row pieces, {row_bytes} bytes apart)",
+                      (lambda p, o: lambda: lib.m2_tile_walk(src.data_ptr(), dst.data_ptr(), batch, rows, row_bytes, p, o, stream()))(piece, in_order)))
+    for name, launch in cases:
+        ms = timed(launch)
+        rows_out.append({"pattern": name, "us": ms * 1e3, "GB/s": moved / (ms * 1e-3) / 1e9})
+    copy, head = rows_out[0], rows_out[3]
+    return dict(metric="HBM rate of a no-arithmetic kernel with the SSD kernels' access pattern", value=head["GB/s"], unit="GB/s",
+                ms_per_step=head["us"] * 1e-3, dtype="u8",
+                config={"workload": f"tile_walk_kernel over x of the c1 shape ({src.numel() / 1e6:.0f} MB read + written), caches cleaned before each launch"},
+                patterns=rows_out,
+                roofline={"bound": "hbm", "achieved": head["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": head["GB/s"] / HBM_PEAK_GBS,
+                          "traffic": None, "algorithmic_bytes_per_step": moved, "kernels": "tile_walk_kernel<8, false>",
+                          "plain_copy_same_size_GBs": copy["GB/s"]})
+
+
 def cpu_model():
     try:
         with open("/proc/cpuinfo") as f:
@@ -556,7 +608,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="all", choices=["all", "ssd", "conv", "glue", "core", "layer", "decode", "model", "copy"])
+    ap.add_argument("--workload", default="all", choices=["all", "ssd", "conv", "glue", "core", "layer", "decode", "model", "copy", "pattern"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--exclude", default="", help="comma-separated workloads to leave out of --workload all (for per-kernel profiles)")
     a = ap.parse_args()
@@ -631,8 +683,10 @@ def main():
         secondary("decode_model", bench_model_step, max(3, a.steps // 4), max(1, a.warmup // 2))
     if wanted("copy"):
         secondary("stream_copy", bench_copy, a.steps, a.warmup)
+    if wanted("pattern"):
+        secondary("access_pattern", bench_access_pattern, a.steps, a.warmup)
     if a.workload not in ("all", "ssd"):
-        key = {"conv": "conv1d", "glue": "mixer_glue", "core": "mixer_core", "layer": "mixer_layer_c3", "decode": "decode", "model": "decode_model", "copy": "stream_copy"}[a.workload]
+        key = {"conv": "conv1d", "glue": "mixer_glue", "core": "mixer_core", "layer": "mixer_layer_c3", "decode": "decode", "model": "decode_model", "copy": "stream_copy", "pattern": "access_pattern"}[a.workload]
         out.update(other.pop(key))
         out.update({"n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "scaling": "weak", "vs_baseline": None, "data": "synthetic"})
         out.setdefault("higher_is_better", True)

@@ -244,9 +244,18 @@ int m2_add_rmsnorm(float* residual, int64_t residual_stride_row, const void* del
  * LDS-staged MFMA tile code the SSD kernels use.  M, N multiples of 128; K multiple of 32.
  * m2_stream_copy: plain copy kernel of `bytes` bytes (multiple of 16), for calibrating
  * bandwidth counters and the achievable-HBM figure.
+ * m2_tile_walk: the access pattern of the SSD kernels without their arithmetic.  src is a (batch, rows, row_bytes)
+ * array; it is read as tiles of 128 rows x piece_bytes (64, 128, 256 or 512: half a head, a head, two, four heads of a
+ * (b, l, h, p) tensor with 128-byte heads) and tile (b, t, u) is written as one contiguous block at
+ * dst + ((b * rows / 128 + t) * (row_bytes / piece_bytes) + u) * 128 * piece_bytes.  in_order != 0: one workgroup per
+ * (b, u) takes its tiles in order, two loads ahead (the state passes' shape); 0: one workgroup per tile.  rows a multiple
+ * of 128, row_bytes a multiple of piece_bytes; dst has the size of src.  Neither has a counterpart in the reference:
+ * they give the rate that the memory system allows a kernel with these streams.
  */
 int m2_mfma_selftest(const void* A, const void* Bt, float* C, int64_t M, int64_t N, int64_t K, int32_t dtype, void* stream);
 int m2_stream_copy(const void* src, void* dst, size_t bytes, void* stream);
+int m2_tile_walk(const void* src, void* dst, int64_t batch, int64_t rows, int64_t row_bytes, int64_t piece_bytes,
+                 int32_t in_order, void* stream);
 
 #ifdef __cplusplus
 }

@@ -60,6 +60,45 @@ mfma_selftest_kernel(const T* __restrict__ A, const T* __restrict__ Bt, float* _
             }
 }
 
+// The HBM streams of the SSD kernels without their arithmetic: a (batch, rows, row_bytes) array is read as tiles of 128
+// rows x `16 PPR` bytes (the rows of one head, or of half a head or of two, of a (b, l, h, p) tensor: short pieces a whole
+// row apart) and every tile is written out as one contiguous block.  IN_ORDER: one workgroup per (batch, column of
+// tiles) takes its tiles one after the other, loading two tiles ahead, as the state passes do; otherwise one workgroup
+// per tile, as in the chunk-parallel kernels.
+template <int PPR, bool IN_ORDER>
+__global__ void __launch_bounds__(256) tile_walk_kernel(const char* __restrict__ src, char* __restrict__ dst, int tiles_down, int64_t row_bytes) {
+    constexpr int ROWS = 128, NX = ROWS * PPR / 256;      // 16-byte pieces per thread per tile
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const int u = blockIdx.x, units = gridDim.x, tid = threadIdx.x;
+    const int64_t b = IN_ORDER ? blockIdx.y : blockIdx.y / tiles_down;
+    const int first = IN_ORDER ? 0 : (int)(blockIdx.y % tiles_down), count = IN_ORDER ? tiles_down : 1;
+    const char* base = src + b * tiles_down * ROWS * row_bytes + (int64_t)u * (PPR * 16);
+    auto load = [&](int t, u32x4* v) {
+        if (t >= first + count) return;
+#pragma unroll
+        for (int i = 0; i < NX; ++i) {
+            const int piece = tid + i * 256, row = piece / PPR, slot = piece % PPR;
+            v[i] = *reinterpret_cast<const u32x4*>(base + ((int64_t)t * ROWS + row) * row_bytes + slot * 16);
+        }
+    };
+    auto store = [&](int t, const u32x4* v) {
+        char* o = dst + ((b * tiles_down + t) * units + u) * (int64_t)(ROWS * PPR * 16);
+#pragma unroll
+        for (int i = 0; i < NX; ++i) *reinterpret_cast<u32x4*>(o + (tid + i * 256) * 16) = v[i];
+    };
+    u32x4 s0[NX], s1[NX];
+    load(first, s0);
+    if (count > 1) load(first + 1, s1);
+    for (int t = first; t < first + count; t += 2) {
+        store(t, s0);
+        load(t + 2, s0);
+        if (t + 1 < first + count) {
+            store(t + 1, s1);
+            load(t + 3, s1);
+        }
+    }
+}
+
 // A workgroup copies blocks of 256 x 4 vectors: four 16-byte loads in flight per lane, each a whole 4 KiB run per wave
 // pair, streamed past the caches on both sides (nothing is read twice).
 __global__ void __launch_bounds__(256) stream_copy_kernel(const floatx4* __restrict__ src, floatx4* __restrict__ dst, size_t n) {
@@ -172,4 +211,32 @@ extern "C" int m2_stream_copy(const void* src, void* dst, size_t bytes, void* st
     if (blocks > 256 * 32) blocks = 256 * 32;
     stream_copy_kernel<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const floatx4*>(src), static_cast<floatx4*>(dst), n);
     return check_launch("stream_copy");
+}
+
+extern "C" int m2_tile_walk(const void* src, void* dst, int64_t batch, int64_t rows, int64_t row_bytes, int64_t piece_bytes,
+                            int32_t in_order, void* stream) {
+    using namespace m2;
+    M2_REQUIRE(src && dst, M2_ERR_NULL, "tile_walk: NULL pointer");
+    M2_REQUIRE(aligned16(src) && aligned16(dst), M2_ERR_ALIGN, "tile_walk: pointers must be multiples of 16 bytes");
+    M2_REQUIRE(batch >= 1 && rows >= 128 && rows % 128 == 0 && row_bytes >= piece_bytes && row_bytes % piece_bytes == 0, M2_ERR_SHAPE,
+               "tile_walk: rows must be a multiple of 128 and row_bytes a multiple of piece_bytes (got rows %lld, row_bytes %lld, piece_bytes %lld)",
+               (long long)rows, (long long)row_bytes, (long long)piece_bytes);
+    const int64_t tiles_down = rows / 128, units = row_bytes / piece_bytes, gy = in_order ? batch : batch * tiles_down;
+    M2_REQUIRE(units <= 0x7fffffff && gy <= 65535 && tiles_down <= 0x7fffffff, M2_ERR_SHAPE, "tile_walk: grid too large");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 grid((unsigned)units, (unsigned)gy);
+    const char* s = static_cast<const char*>(src);
+    char* d = static_cast<char*>(dst);
+#define M2_WALK(PPR) \
+    do { if (in_order) tile_walk_kernel<PPR, true><<<grid, 256, 0, st>>>(s, d, (int)tiles_down, row_bytes); \
+         else tile_walk_kernel<PPR, false><<<grid, 256, 0, st>>>(s, d, (int)tiles_down, row_bytes); } while (0)
+    switch (piece_bytes) {
+        case 64: M2_WALK(4); break;
+        case 128: M2_WALK(8); break;
+        case 256: M2_WALK(16); break;
+        case 512: M2_WALK(32); break;
+        default: return fail(M2_ERR_SHAPE, "tile_walk: piece_bytes must be 64, 128, 256 or 512 (got %lld)", (long long)piece_bytes);
+    }
+#undef M2_WALK
+    return check_launch("tile_walk");
 }

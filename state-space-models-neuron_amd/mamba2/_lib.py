@@ -94,6 +94,7 @@ SYMBOLS = {
     "m2_add_rmsnorm": (C.c_int, [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _i64, C.c_float, _i32, _vp]),
     "m2_mfma_selftest": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp]),
     "m2_stream_copy": (C.c_int, [_vp, _vp, _sz, _vp]),
+    "m2_tile_walk": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _i64, C.c_int32, _vp]),
 }
 
 _lib = None

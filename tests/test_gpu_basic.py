@@ -33,6 +33,26 @@ def test_mfma_tile_selftest(lib, dtype):
     assert rel_err(Cm.cpu(), ref) < (1e-5 if dtype == torch.float32 else 1e-5)   # exact products, fp32 accumulation
 
 
+# ----------------------------------------------------------------------------- memory probes
+def test_stream_copy_and_tile_walk_are_exact(lib):
+    """The measurement probes move bytes and nothing else: the copy is the identity, the tile walk a re-tiling."""
+    from mamba2 import _lib
+    batch, rows, row_bytes = 2, 384, 1024
+    g = torch.Generator().manual_seed(5)
+    src = torch.randint(0, 256, (batch, rows, row_bytes), generator=g, dtype=torch.uint8).to(DEV)
+    dst = torch.zeros_like(src)
+    _lib.check(lib.m2_stream_copy(_lib.ptr(src), _lib.ptr(dst), src.numel(), _lib.stream_ptr()), "copy")
+    assert torch.equal(dst, src)
+    for piece in (64, 128, 256, 512):
+        units = row_bytes // piece
+        want = src.view(batch, rows // 128, 128, units, piece).permute(0, 1, 3, 2, 4).contiguous().view(-1)
+        for in_order in (1, 0):
+            dst.zero_()
+            _lib.check(lib.m2_tile_walk(_lib.ptr(src), _lib.ptr(dst), batch, rows, row_bytes, piece, in_order, _lib.stream_ptr()), "walk")
+            assert torch.equal(dst.view(-1), want), (piece, in_order)
+    assert lib.m2_tile_walk(_lib.ptr(src), _lib.ptr(dst), batch, rows, row_bytes, 96, 1, _lib.stream_ptr()) != 0      # refused, not run
+
+
 # ----------------------------------------------------------------------------- conv1d
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("b,l,C", [(2, 256, 512), (3, 100, 264), (1, 5, 8), (2, 33, 7), (1, 1, 64), (1, 2, 16), (1, 3, 16)])
