@@ -257,6 +257,31 @@ def greedy_generate(model: "Mamba2ForCausalLM", input_ids, max_new_tokens: int, 
     return torch.cat(out, dim=1)
 
 
+class _TunedGemms:
+    """torch.cuda.tunable switched on for a stretch of code and put back afterwards.  Results go to a file in the
+    temporary directory unless the caller has chosen one (TunableOp writes its table when the process ends)."""
+
+    def __init__(self):
+        import os
+        import tempfile
+        import torch.cuda.tunable as tunable
+        self.t = tunable
+        self.was_enabled, self.was_tuning = tunable.is_enabled(), tunable.tuning_is_enabled()
+        if not self.was_enabled and not os.environ.get("PYTORCH_TUNABLEOP_FILENAME"):
+            tunable.set_filename(os.path.join(tempfile.gettempdir(), f"mamba2_tunableop_{os.getpid()}.csv"))
+
+    def start_tuning(self):
+        self.t.enable(True)
+        self.t.tuning_enable(True)
+
+    def stop_tuning(self):
+        self.t.tuning_enable(False)
+
+    def restore(self):
+        self.t.tuning_enable(self.was_tuning)
+        self.t.enable(self.was_enabled)
+
+
 class GraphedStep:
     """``Mamba2ForCausalLM.step`` for one batch size, captured once into a HIP graph and replayed per token.
 
@@ -267,25 +292,41 @@ class GraphedStep:
     addresses, and for a model kept in bfloat16 the fp32 copies of the small per-head and norm parameters made before the
     capture): build a new object after loading other weights.  ``cache_params`` may be reset or refilled by a prefill
     between replays.  The states advanced by the warm-up and capture runs are restored before ``__init__`` returns.
+
+    ``tune_gemms=True`` lets torch's TunableOp time the BLAS libraries' solutions for the step's projection shapes (in_proj,
+    out_proj, LM head: 128-row products for which the libraries' default choices are 15-25 % off their best) during the
+    warm-up and captures the chosen ones; the process-wide TunableOp switches are put back afterwards, the graph keeps the
+    kernels it captured.  The chosen solutions may round differently from the default ones, so replays then agree with the
+    eager step to bf16 accuracy, not bit for bit.
     """
 
-    def __init__(self, model: Mamba2ForCausalLM, cache_params: Mamba2Cache, batch_size: int, warmup: int = 2):
+    def __init__(self, model: Mamba2ForCausalLM, cache_params: Mamba2Cache, batch_size: int, warmup: int = 2,
+                 tune_gemms: bool = False):
         dev = model.device
         if dev.type != "cuda":
             raise RuntimeError("GraphedStep needs the model on a GPU device; there is no CPU path")
         self.model, self.cache = model, cache_params
         self.input_ids = torch.zeros(batch_size, 1, dtype=torch.long, device=dev)
         keep = [t.clone() for t in cache_params.conv_states + cache_params.ssm_states]
+        tun = _TunedGemms() if tune_gemms else None
         side = torch.cuda.Stream(device=dev)
         side.wait_stream(torch.cuda.current_stream(dev))
         with torch.no_grad(), torch.cuda.stream(side):
+            if tun:
+                tun.start_tuning()              # the first warm-up step times the libraries' solutions for its three GEMM shapes
             for _ in range(warmup):             # lazily created workspaces and library handles exist before the capture
                 model.step(self.input_ids, cache_params)
+            if tun:
+                tun.stop_tuning()               # (no timing runs inside the capture: the chosen solutions are looked up)
         torch.cuda.current_stream(dev).wait_stream(side)
         torch.cuda.synchronize(dev)
         self.graph = torch.cuda.CUDAGraph()
-        with torch.no_grad(), torch.cuda.graph(self.graph):
-            self.logits = model.step(self.input_ids, cache_params)
+        try:
+            with torch.no_grad(), torch.cuda.graph(self.graph):
+                self.logits = model.step(self.input_ids, cache_params)
+        finally:
+            if tun:
+                tun.restore()
         for t, k in zip(cache_params.conv_states + cache_params.ssm_states, keep):
             t.copy_(k)
 

@@ -237,6 +237,38 @@ def test_graphed_step_replays_equal_eager_steps(dtype):
         assert torch.equal(step(ids[:, 9:10]), m.step(ids[:, 9:10], cache_e))
 
 
+def test_graphed_step_with_tuned_gemms_agrees_with_eager():
+    """tune_gemms: the captured projections may be other library solutions than the eager ones; replays agree with the eager
+    step to bf16 accuracy, the process-wide TunableOp switches are back where they were, and nothing keeps tuning."""
+    import torch.cuda.tunable as tunable
+    from mamba2.mamba2_mixer import Mamba2Cache
+    from mamba2.modeling_mamba2 import GraphedStep
+    dtype = torch.bfloat16
+    cfg, m = _model(dtype, layers=2)
+    b = 4
+    ids = torch.randint(0, cfg.vocab_size, (b, 30), generator=torch.Generator().manual_seed(9)).to(DEV)
+    cache_g = Mamba2Cache(cfg, b, dtype=dtype, device=DEV, conv_width=3)
+    cache_e = Mamba2Cache(cfg, b, dtype=dtype, device=DEV, conv_width=3)
+    with torch.no_grad():
+        m(input_ids=ids[:, :9], cache_params=cache_g, use_cache=True)
+        m(input_ids=ids[:, :9], cache_params=cache_e, use_cache=True)
+    before = (tunable.is_enabled(), tunable.tuning_is_enabled())
+    step = GraphedStep(m, cache_g, b, tune_gemms=True)
+    assert (tunable.is_enabled(), tunable.tuning_is_enabled()) == before
+    for i in range(cfg.num_hidden_layers):          # capture, tuning runs and warm-up left the states where they were
+        assert torch.equal(cache_g.ssm_states[i], cache_e.ssm_states[i]) and torch.equal(cache_g.conv_states[i], cache_e.conv_states[i])
+    for t in range(9, 30):
+        got = step(ids[:, t:t + 1]).clone()
+        torch.cuda.synchronize()
+        with torch.no_grad():
+            ref = m.step(ids[:, t:t + 1], cache_e)
+        torch.cuda.synchronize()
+        g_, r_ = got.double(), ref.double()
+        assert ((g_ - r_).norm() / r_.norm()).item() < 2e-2, t          # two bf16 evaluations of the same step
+    for i in range(cfg.num_hidden_layers):
+        assert rel_err(cache_g.ssm_states[i], cache_e.ssm_states[i]) < 2e-2
+
+
 def test_decode_step_softplus_inside_matches_softplus_outside():
     """m2_decode_step with dt_bias (raw dt) against the same step fed softplus(dt + dt_bias) computed by the oracle."""
     from mamba2.mamba2_kernel_inference import mamba2_kernel_inference
