@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X Mamba-2 mixer hot path.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|ssd|conv|glue|core|layer|decode|model|copy] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|ssd|conv|glue|core|layer|decode|model|copy|pattern] [--no-cpu] [--no-gemm-tuning]
 
 One "step" is one pass of the hot path over one batch of synthetic input, inputs resident in HBM:
   ssd    : SSD chunked scan fwd+bwd, bf16, 2.7B shape (b4, l2048, h80, p64, n128, g1, chunk 128)   <- headline
@@ -398,7 +398,7 @@ def bench_decode(steps, warmup):
                           "algorithmic_bytes_per_step": bytes_, "kernels": "decode_conv_kernel + decode_ssm_kernel, 64 launches each"})
 
 
-def bench_model_step(steps, warmup):
+def bench_model_step(steps, warmup, tune_gemms=True):
     """One decode step of the whole 2.7B-shaped model (embedding, 64 x [RMSNorm, in_proj, decode kernels, gated norm,
     out_proj, residual], final norm, LM head) at batch 128: eager launches and the same step replayed from one HIP graph."""
     import torch
@@ -423,7 +423,7 @@ def bench_model_step(steps, warmup):
             model.step(ids, cache)
 
     wall_e, per_e = event_time_ms(eager, steps, warmup)
-    graphed = GraphedStep(model, cache, b, tune_gemms=True)      # the serving form: the libraries' best solutions for the three GEMM shapes
+    graphed = GraphedStep(model, cache, b, tune_gemms=tune_gemms)      # the serving form: the libraries' best solutions for the three GEMM shapes
     wall_g, per_g = event_time_ms(lambda: graphed(ids), steps, warmup)
     ms_e, ms_g = sum(per_e) / len(per_e), sum(per_g) / len(per_g)
     # bytes a step has to move: every layer's states read and written, every weight but the embedding table read once
@@ -436,7 +436,7 @@ def bench_model_step(steps, warmup):
                 config={"workload": "Mamba2ForCausalLM.step, d_model 2560, 64 layers, h80 p64 n128 g1, vocab 50288, b128, conv state W3"},
                 roofline={"bound": "hbm", "achieved": bytes_ / (ms_g * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": bytes_ / (ms_g * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_step": bytes_,
-                          "kernels": "one graph replay: projections (rocBLAS / hipBLASLt solutions chosen by torch TunableOp during the graph's warm-up; the eager figure uses the libraries' defaults) + decode_conv/decode_ssm/rmsnorm_gated kernels + torch elementwise"})
+                          "kernels": "one graph replay: projections (" + ("rocBLAS / hipBLASLt solutions chosen by torch TunableOp during the graph's warm-up; the eager figure uses the libraries' defaults" if tune_gemms else "the BLAS libraries' default solutions") + ") + decode_conv/decode_ssm/rmsnorm_gated kernels + torch elementwise"})
 
 
 def bench_copy(steps, warmup):
@@ -610,6 +610,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all", choices=["all", "ssd", "conv", "glue", "core", "layer", "decode", "model", "copy", "pattern"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-gemm-tuning", action="store_true",
+                    help="model workload: capture the step with the BLAS libraries' default solutions (for kernel traces: the tuning runs would fill them)")
     ap.add_argument("--exclude", default="", help="comma-separated workloads to leave out of --workload all (for per-kernel profiles)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -680,7 +682,7 @@ def main():
     if wanted("decode"):
         secondary("decode", bench_decode, max(3, a.steps // 4), max(1, a.warmup // 2))
     if wanted("model"):
-        secondary("decode_model", bench_model_step, max(3, a.steps // 4), max(1, a.warmup // 2))
+        secondary("decode_model", bench_model_step, max(3, a.steps // 4), max(1, a.warmup // 2), not a.no_gemm_tuning)
     if wanted("copy"):
         secondary("stream_copy", bench_copy, a.steps, a.warmup)
     if wanted("pattern"):
