@@ -11,7 +11,7 @@ class Mamba2Config:
                  hidden_act="silu", initializer_range=0.1, residual_in_fp32=True, time_step_rank="auto",
                  time_step_min=0.001, time_step_max=0.1, time_step_floor=1e-4, time_step_limit=(0.0, float("inf")),
                  rescale_prenorm_residual=False, use_cache=True, rms_norm=True, rmsnorm_within_groups=True, chunk_size=256,
-                 tie_word_embeddings=False, sequence_parallel_enabled=False, dtype=None, **kwargs):
+                 tie_word_embeddings=False, sequence_parallel_enabled=False, dtype=None, recompute_core=False, **kwargs):
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.state_size = state_size
@@ -38,6 +38,10 @@ class Mamba2Config:
         self.chunk_size = chunk_size
         self.time_step_limit = tuple(time_step_limit)
         self.tie_word_embeddings = tie_word_embeddings
+        # False: the fused core keeps its conv output, scan output and chunk states for the backward (288 GB of HBM make that
+        # cheaper than a second forward); True: only the inputs are kept and the backward recomputes, as the reference's
+        # mixer does (mamba2_mixer.py:229)
+        self.recompute_core = recompute_core
         self.sequence_parallel_enabled = sequence_parallel_enabled
         self.dtype = dtype
         for k, v in kwargs.items():

@@ -18,7 +18,7 @@ from torch import nn
 
 from .configuration_mamba2 import Mamba2Config
 from .conv1d_grouped import ConvNKI
-from .fused_kernel import mamba2_fused_kernel, mamba2_fused_prefill
+from .fused_kernel import mamba2_fused_kernel, mamba2_fused_kernel_with_caching, mamba2_fused_prefill
 from .mamba2_kernel_inference import mamba2_kernel_inference
 from . import glue
 
@@ -127,6 +127,7 @@ class Mamba2Mixer(nn.Module):
         self.num_heads_tp = self.num_heads
         self.conv_dim_tp = self.conv_dim
         self._fp32_params = None
+        self.recompute_core = bool(getattr(config, "recompute_core", False))
 
     def _inference_params(self):
         """fp32 (A, D, dt_bias) as the decode kernel takes them, rebuilt only when a parameter changed."""
@@ -155,8 +156,9 @@ class Mamba2Mixer(nn.Module):
             return self.out_proj(scan_output)
         A = -torch.exp(self.A_log.float())
         zxBCdt = self.in_proj(hidden_states)
-        scan_output = mamba2_fused_kernel(zxBCdt, A, self.D, self.conv1d.weight, self.conv1d.bias, self.dt_bias, self.norm.weight,
-                                          self.n_groups_tp, self.ssm_state_size, self.intermediate_size_tp, self.head_dim)
+        core = mamba2_fused_kernel if self.recompute_core else mamba2_fused_kernel_with_caching
+        scan_output = core(zxBCdt, A, self.D, self.conv1d.weight, self.conv1d.bias, self.dt_bias, self.norm.weight,
+                           self.n_groups_tp, self.ssm_state_size, self.intermediate_size_tp, self.head_dim)
         return self.out_proj(scan_output)
 
     def forward(self, hidden_states, cache_params: Optional[Mamba2Cache] = None,

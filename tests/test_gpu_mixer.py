@@ -117,8 +117,10 @@ def test_mixer_parameter_names_and_shapes():
     assert names["norm.weight"].shape == (d_inner,)
 
 
-def test_mixer_forward_backward_matches_oracle():
+@pytest.mark.parametrize("recompute", [False, True])
+def test_mixer_forward_backward_matches_oracle(recompute):
     cfg, m = _mixer(torch.float32)
+    m.recompute_core = recompute            # False (default): the core's activations are kept; True: the reference's recompute
     x = torch.randn(2, 256, 128, generator=torch.Generator().manual_seed(1))
     xd = x.to(DEV).requires_grad_(True)
     y = m(xd)
