@@ -428,7 +428,14 @@ def bench_model_step(steps, warmup, tune_gemms=True):
             model.step(ids, cache)
 
     wall_e, per_e = event_time_ms(eager, steps, warmup)
-    graphed = GraphedStep(model, cache, b, tune_gemms=tune_gemms)      # the serving form: the libraries' best solutions for the three GEMM shapes
+    try:
+        graphed = GraphedStep(model, cache, b, tune_gemms=tune_gemms)      # the serving form: the libraries' best solutions for the three GEMM shapes
+    except Exception as e:      # noqa: BLE001  (a torch build without TunableOp: the default solutions, and the line says so)
+        if not tune_gemms:
+            raise
+        print(f"bench: GEMM tuning unavailable ({type(e).__name__}: {e}); capturing the default solutions", file=sys.stderr)
+        tune_gemms = False
+        graphed = GraphedStep(model, cache, b)
     wall_g, per_g = event_time_ms(lambda: graphed(ids), steps, warmup)
     ms_e, ms_g = sum(per_e) / len(per_e), sum(per_g) / len(per_g)
     # bytes a step has to move: every layer's states read and written, every weight but the embedding table read once

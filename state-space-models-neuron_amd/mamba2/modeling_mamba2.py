@@ -309,19 +309,19 @@ class GraphedStep:
         self.input_ids = torch.zeros(batch_size, 1, dtype=torch.long, device=dev)
         keep = [t.clone() for t in cache_params.conv_states + cache_params.ssm_states]
         tun = _TunedGemms() if tune_gemms else None
-        side = torch.cuda.Stream(device=dev)
-        side.wait_stream(torch.cuda.current_stream(dev))
-        with torch.no_grad(), torch.cuda.stream(side):
-            if tun:
-                tun.start_tuning()              # the first warm-up step times the libraries' solutions for its three GEMM shapes
-            for _ in range(warmup):             # lazily created workspaces and library handles exist before the capture
-                model.step(self.input_ids, cache_params)
-            if tun:
-                tun.stop_tuning()               # (no timing runs inside the capture: the chosen solutions are looked up)
-        torch.cuda.current_stream(dev).wait_stream(side)
-        torch.cuda.synchronize(dev)
-        self.graph = torch.cuda.CUDAGraph()
         try:
+            side = torch.cuda.Stream(device=dev)
+            side.wait_stream(torch.cuda.current_stream(dev))
+            with torch.no_grad(), torch.cuda.stream(side):
+                if tun:
+                    tun.start_tuning()          # the first warm-up step times the libraries' solutions for its three GEMM shapes
+                for _ in range(warmup):         # lazily created workspaces and library handles exist before the capture
+                    model.step(self.input_ids, cache_params)
+                if tun:
+                    tun.stop_tuning()           # (no timing runs inside the capture: the chosen solutions are looked up)
+            torch.cuda.current_stream(dev).wait_stream(side)
+            torch.cuda.synchronize(dev)
+            self.graph = torch.cuda.CUDAGraph()
             with torch.no_grad(), torch.cuda.graph(self.graph):
                 self.logits = model.step(self.input_ids, cache_params)
         finally:
